@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Headline benchmark: SGNS training step (word2vecPos + word2vecNeg) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one minibatch of the headline configuration (vocab 1M, dim 300, fp32, 1M tokens from a
+Zipf(1.0) stream, window half-width 5, 5 negatives per positive drawn from unigram^0.75, groups of
+5 contexts) pushed through the two update operators.  Index arrays and tables are resident in HBM
+before the timed region starts.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: vocab, dim, tokens per minibatch, window half-width, nneg, nreuse, zipf exponent
+    "sgns_v1m_d300_w5_neg5_fp32": dict(vocab=1_000_000, dim=300, tokens=1_000_000, skip=5, nneg=5,
+                                       nreuse=5, zipf=1.0),
+    "sgns_v1m_d512_w10_neg15_fp32": dict(vocab=1_000_000, dim=512, tokens=500_000, skip=10,
+                                         nneg=15, nreuse=5, zipf=1.0),
+    "sgns_v10k_d100_w5_neg5_fp32": dict(vocab=10_000, dim=100, tokens=100_000, skip=5, nneg=5,
+                                        nreuse=5, zipf=1.0),
+}
+
+
+def make_minibatch(cfg, index, zcdf, ncdf):
+    """Index arrays of minibatch `index` of the stream (seeded, reproducible)."""
+    from bidmach_amd import corpus
+    n = cfg["tokens"]
+    W = corpus.zipf_stream(n, cfg["vocab"], cfg["zipf"], seed=1234 + index, cdf=zcdf)
+    rng = np.random.Generator(np.random.PCG64(99 + index))
+    LB, UB = corpus.window_bounds(n, cfg["skip"], rng)
+    WA, WB, G = corpus.negative_groups(W, LB, UB, cfg["nneg"], cfg["nreuse"], rng, neg_cdf=ncdf)
+    pairs, centres = corpus.count_pairs(W, LB, UB)
+    return dict(W=W, LB=LB, UB=UB, WA=WA, WB=WB, G=G, pairs=pairs, centres=centres)
+
+
+def algorithmic_bytes(cfg, mb):
+    """Gather-scatter model: one read and one write of every column a work unit touches, plus the
+    index arrays.  Pos: 2*C*(centres + pairs) + 12*N.  Neg: 2*C*G*(nwa+nwb) + 4*G*(nwa+nwb)."""
+    C = cfg["dim"] * 4
+    pos = 2 * C * (mb["centres"] + mb["pairs"]) + 12 * cfg["tokens"]
+    k = cfg["nneg"] + cfg["nreuse"]
+    neg = 2 * C * mb["G"] * k + 4 * mb["G"] * k
+    return pos, neg
+
+
+def cpu_baseline(cfg, mb, lr_pos, lr_neg, vexp, threads):
+    """Times the C oracle (a port of the reference CPU path, built with the reference's flags) on
+    one full minibatch of the same workload, on this machine's host cores."""
+    from bidmach_amd import corpus
+    from oracle.cpumach import CPUMACH
+    d, n = cfg["dim"], cfg["tokens"]
+    B, A = corpus.init_tables(cfg["vocab"], d, seed=42)
+    # warm-up on a slice so page faults and thread start-up stay out of the timing
+    m = min(n, 20000)
+    CPUMACH.word2vecPos(d, m, cfg["skip"], mb["W"][:m].copy(), mb["LB"][:m].copy(),
+                        mb["UB"][:m].copy(), A, B, lr_pos, vexp, threads)
+    t0 = time.perf_counter()
+    CPUMACH.word2vecPos(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr_pos, vexp, threads)
+    CPUMACH.word2vecNeg(d, mb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"], mb["WB"], A, B, lr_neg,
+                        vexp, threads)
+    dt = time.perf_counter() - t0
+    return n / dt, dt
+
+
+def host_threads():
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        n = min(n, int(env))
+    return max(1, n)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="sgns_v1m_d300_w5_neg5_fp32", choices=sorted(WORKLOADS))
+    ap.add_argument("--vexp", type=float, default=0.0)
+    ap.add_argument("--lrate", type=float, default=0.025)
+    ap.add_argument("--distinct", type=int, default=8,
+                    help="number of distinct minibatches generated; steps cycle through them")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); "
+                 "run it with --gpus 1")
+
+    import torch
+    from bidmach_amd import corpus
+    from bidmach_amd.cumach import CUMACH, Timer, check, synchronize
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    cfg = WORKLOADS[args.workload]
+    d, V, n = cfg["dim"], cfg["vocab"], cfg["tokens"]
+    K, Wm = args.steps, args.warmup
+
+    t_prep = time.perf_counter()
+    zcdf = corpus.zipf_cdf(V, cfg["zipf"])
+    ncdf = corpus.unigram_pow_cdf(V, cfg["zipf"], 0.75)
+    ndistinct = max(1, min(args.distinct, K + Wm))
+    host_mbs = [make_minibatch(cfg, i, zcdf, ncdf) for i in range(ndistinct)]
+    dev_mbs = []
+    for mb in host_mbs:
+        dev_mbs.append({k: torch.from_numpy(mb[k]).cuda() for k in ("W", "LB", "UB", "WA", "WB")})
+    Bh, Ah = corpus.init_tables(V, d, seed=42)
+    A = torch.from_numpy(Ah).cuda()
+    B = torch.from_numpy(Bh).cuda()
+    del Ah, Bh
+    torch.cuda.synchronize()
+    t_prep = time.perf_counter() - t_prep
+
+    total = K + Wm
+
+    def lrate(step):   # linear decay over the run, floor at 1e-4 of the start
+        return max(args.lrate * (1.0 - step / float(max(total, 1))), args.lrate * 1e-4)
+
+    def step(s, timers=None):
+        mb, hmb = dev_mbs[s % ndistinct], host_mbs[s % ndistinct]
+        lr = lrate(s)
+        if timers:
+            timers[0].start()
+        check(CUMACH.word2vecPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr,
+                                      args.vexp), "word2vecPos")
+        if timers:
+            timers[0].stop()
+            timers[1].start()
+        check(CUMACH.word2vecNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"], mb["WB"],
+                                      A, B, lr / cfg["nneg"], args.vexp), "word2vecNeg")
+        if timers:
+            timers[1].stop()
+
+    for s in range(Wm):
+        step(s)
+    synchronize()
+    torch.cuda.synchronize()
+
+    timers = [(Timer(), Timer()) for _ in range(K)]
+    t0 = time.perf_counter()
+    for s in range(K):
+        step(Wm + s, timers[s])
+    synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    pos_ms = [t[0].elapsed_ms() for t in timers]
+    neg_ms = [t[1].elapsed_ms() for t in timers]
+    pos_b, neg_b = zip(*[algorithmic_bytes(cfg, host_mbs[(Wm + s) % ndistinct]) for s in range(K)])
+    avg_pos_ms, avg_neg_ms = float(np.mean(pos_ms)), float(np.mean(neg_ms))
+    avg_pos_b, avg_neg_b = float(np.mean(pos_b)), float(np.mean(neg_b))
+    pos_gbps = avg_pos_b / (avg_pos_ms * 1e-3) / 1e9
+    neg_gbps = avg_neg_b / (avg_neg_ms * 1e-3) / 1e9
+    step_gbps = (avg_pos_b + avg_neg_b) / ((avg_pos_ms + avg_neg_ms) * 1e-3) / 1e9
+
+    assert bool(torch.isfinite(A).all()) and bool(torch.isfinite(B).all()), "tables diverged"
+
+    words_per_s = K * n / elapsed
+    out = {
+        "metric": "updated words/sec, SGNS V=1M d=300 w=5 neg=5 fp32"
+                  if args.workload == "sgns_v1m_d300_w5_neg5_fp32"
+                  else "updated words/sec, " + args.workload,
+        "value": words_per_s,
+        "unit": "words/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": Wm,
+        "ms_per_step": elapsed / K * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "vocab": V, "dim": d, "tokens_per_minibatch": n,
+                   "window": cfg["skip"], "nneg": cfg["nneg"], "nreuse": cfg["nreuse"],
+                   "zipf_s": cfg["zipf"], "vexp": args.vexp, "lrate": args.lrate,
+                   "distinct_minibatches": ndistinct,
+                   "pairs_per_minibatch": int(np.mean([m["pairs"] for m in host_mbs])),
+                   "groups_per_minibatch": int(np.mean([m["G"] for m in host_mbs]))},
+        # the negative pass moves ~63% of the step's algorithmic bytes: it is the dominant kernel
+        "roofline": {"bound": "hbm", "kernel": "neg_kernel", "achieved": neg_gbps,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": neg_gbps / HBM_PEAK_GBPS,
+                     "traffic": None, "algorithmic_bytes_per_launch": avg_neg_b,
+                     "avg_launch_ms": avg_neg_ms},
+        "kernels": {
+            "pos_kernel": {"avg_launch_ms": avg_pos_ms, "algorithmic_bytes_per_launch": avg_pos_b,
+                           "achieved_GBps": pos_gbps, "frac": pos_gbps / HBM_PEAK_GBPS},
+            "neg_kernel": {"avg_launch_ms": avg_neg_ms, "algorithmic_bytes_per_launch": avg_neg_b,
+                           "achieved_GBps": neg_gbps, "frac": neg_gbps / HBM_PEAK_GBPS},
+            "step": {"achieved_GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
+                     "kernel_ms": avg_pos_ms + avg_neg_ms},
+        },
+        "host_prep_s": t_prep,
+    }
+
+    if not args.no_cpu_baseline:
+        threads = host_threads()
+        cpu_wps, cpu_dt = cpu_baseline(cfg, host_mbs[0], args.lrate, args.lrate / cfg["nneg"],
+                                       args.vexp, threads)
+        out["cpu_baseline"] = {"value": cpu_wps, "unit": "words/s", "cores": threads,
+                               "kind": "port",
+                               "sample": "one full minibatch (%d tokens) of the same workload, "
+                                         "pos+neg, %.1f s wall" % (n, cpu_dt),
+                               "gpu_over_cpu": words_per_s / cpu_wps}
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,56 @@
+"""Builds the HIP shared library in-tree with hipcc for gfx950.
+
+    python -m bidmach_amd.build
+
+Objects go to bidmach_amd/csrc/_obj/, the library to bidmach_amd/lib/.  The library name follows
+the reference's artefact naming (jni/src/Makefile:11-21: libbidmachcuda-linux-x86_64.so).
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "_obj")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_NAME = "libbidmachhip-linux-x86_64.so"
+LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
+
+SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_api.hip"]
+
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+    "-munsafe-fp-atomics",
+    # keep the compiler from forming packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _hipcc():
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(src, extra):
+    out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc()] + HIPCC_FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", out]
+    subprocess.check_call(cmd)
+    return out
+
+
+def build(extra_flags=(), verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    extra = list(extra_flags)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(lambda s: _compile(s, extra), SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    subprocess.check_call(cmd)
+    if verbose:
+        print("built", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build(sys.argv[1:])

@@ -1,0 +1,254 @@
+// C ABI of the SGNS library: argument checks, per-thread stream and Eval scratch, launch,
+// and the synchronous/asynchronous forms of the four operators.
+#include "../../include/bidmach_w2v.h"
+
+#include <atomic>
+#include <cstring>
+
+#include "w2v_internal.h"
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+
+struct ThreadState {
+  hipStream_t stream = nullptr;
+  double* partials[kMaxDevices] = {};
+  int64_t capacity[kMaxDevices] = {};
+};
+
+thread_local ThreadState t_state;
+
+std::atomic<double> g_eval_floor{1.0e-40};
+
+// Per-thread, per-device buffer of per-block partial sums for the Eval kernels.  It only grows.
+hipError_t eval_scratch(int64_t need, double** out) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  ThreadState& ts = t_state;
+  if (ts.capacity[dev] < need) {
+    if (ts.partials[dev] != nullptr) {
+      err = hipStreamSynchronize(ts.stream);
+      if (err != hipSuccess) return err;
+      err = hipFree(ts.partials[dev]);
+      ts.partials[dev] = nullptr;
+      ts.capacity[dev] = 0;
+      if (err != hipSuccess) return err;
+    }
+    int64_t cap = 4096;
+    while (cap < need) cap *= 2;
+    err = hipMalloc(reinterpret_cast<void**>(&ts.partials[dev]), (size_t)cap * sizeof(double));
+    if (err != hipSuccess) {
+      ts.partials[dev] = nullptr;
+      return err;
+    }
+    ts.capacity[dev] = cap;
+  }
+  *out = ts.partials[dev];
+  return hipSuccess;
+}
+
+bool bad_common(int nrows, int ncols) {
+  return nrows <= 0 || nrows > w2v::max_rows() || ncols < 0;
+}
+
+int finish(hipError_t launch_err, bool sync) {
+  if (launch_err != hipSuccess) return (int)launch_err;
+  if (sync) {
+    hipError_t err = hipStreamSynchronize(t_state.stream);
+    if (err != hipSuccess) return (int)err;
+    return (int)hipGetLastError();
+  }
+  return 0;
+}
+
+int pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, float* B, float lrate,
+             float vexp, bool sync) {
+  if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp), sync);
+}
+
+int neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
+             float lrate, float vexp, bool sync) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb())
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(
+      w2v::launch_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp), sync);
+}
+
+int eval_pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, float* B, float* r32,
+                  double* r64, bool sync) {
+  if (bad_common(nrows, ncols) || (!r32 && !r64)) return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  double* partials = nullptr;
+  hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_eval_pos(t_state.stream, nrows, ncols, W, LB, UB, A, B,
+                                     g_eval_floor.load(), partials, r32, r64),
+                sync);
+}
+
+int eval_neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
+                  float* r32, double* r64, bool sync) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || (!r32 && !r64))
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  double* partials = nullptr;
+  hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+                                     g_eval_floor.load(), partials, r32, r64),
+                sync);
+}
+
+struct Timer {
+  hipEvent_t start;
+  hipEvent_t stop;
+};
+
+}  // namespace
+
+extern "C" {
+
+int word2vecPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
+                float lrate, float vexp) {
+  (void)shift;
+  return pos_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, true);
+}
+
+int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
+                float lrate, float vexp) {
+  return neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, true);
+}
+
+int word2vecEvalPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
+                    float* Retval) {
+  (void)shift;
+  return eval_pos_impl(nrows, ncols, W, LB, UB, A, B, Retval, nullptr, true);
+}
+
+int word2vecEvalNeg(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
+                    float* Retval) {
+  return eval_neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, Retval, nullptr, true);
+}
+
+int word2vecEvalPosF64(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A,
+                       float* B, double* Retval) {
+  (void)shift;
+  return eval_pos_impl(nrows, ncols, W, LB, UB, A, B, nullptr, Retval, true);
+}
+
+int word2vecEvalNegF64(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A,
+                       float* B, double* Retval) {
+  return eval_neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, nullptr, Retval, true);
+}
+
+int word2vecPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
+                     float lrate, float vexp) {
+  (void)shift;
+  return pos_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, false);
+}
+
+int word2vecNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
+                     float lrate, float vexp) {
+  return neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, false);
+}
+
+int word2vecEvalPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A,
+                         float* B, float* Retval) {
+  (void)shift;
+  return eval_pos_impl(nrows, ncols, W, LB, UB, A, B, Retval, nullptr, false);
+}
+
+int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A,
+                         float* B, float* Retval) {
+  return eval_neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, Retval, nullptr, false);
+}
+
+void w2v_set_eval_floor(double floor_value) { g_eval_floor.store(floor_value); }
+double w2v_get_eval_floor(void) { return g_eval_floor.load(); }
+
+int w2v_set_stream(void* stream) {
+  t_state.stream = reinterpret_cast<hipStream_t>(stream);
+  return 0;
+}
+void* w2v_get_stream(void) { return reinterpret_cast<void*>(t_state.stream); }
+int w2v_synchronize(void) { return (int)hipStreamSynchronize(t_state.stream); }
+
+int w2v_max_rows(void) { return w2v::max_rows(); }
+int w2v_max_nwb(void) { return w2v::max_nwb(); }
+
+int w2v_malloc(void** dev_ptr, size_t bytes) {
+  if (!dev_ptr) return (int)hipErrorInvalidValue;
+  return (int)hipMalloc(dev_ptr, bytes);
+}
+int w2v_free(void* dev_ptr) { return (int)hipFree(dev_ptr); }
+int w2v_memcpy_h2d(void* dev_dst, const void* host_src, size_t bytes) {
+  hipError_t err = hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, t_state.stream);
+  if (err != hipSuccess) return (int)err;
+  return (int)hipStreamSynchronize(t_state.stream);
+}
+int w2v_memcpy_d2h(void* host_dst, const void* dev_src, size_t bytes) {
+  hipError_t err = hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, t_state.stream);
+  if (err != hipSuccess) return (int)err;
+  return (int)hipStreamSynchronize(t_state.stream);
+}
+int w2v_memset(void* dev_ptr, int value, size_t bytes) {
+  hipError_t err = hipMemsetAsync(dev_ptr, value, bytes, t_state.stream);
+  if (err != hipSuccess) return (int)err;
+  return (int)hipStreamSynchronize(t_state.stream);
+}
+
+int w2v_timer_create(void** timer) {
+  if (!timer) return (int)hipErrorInvalidValue;
+  Timer* t = new (std::nothrow) Timer();
+  if (!t) return (int)hipErrorOutOfMemory;
+  hipError_t err = hipEventCreate(&t->start);
+  if (err != hipSuccess) {
+    delete t;
+    return (int)err;
+  }
+  err = hipEventCreate(&t->stop);
+  if (err != hipSuccess) {
+    (void)hipEventDestroy(t->start);
+    delete t;
+    return (int)err;
+  }
+  *timer = t;
+  return 0;
+}
+int w2v_timer_destroy(void* timer) {
+  if (!timer) return 0;
+  Timer* t = static_cast<Timer*>(timer);
+  hipError_t e1 = hipEventDestroy(t->start);
+  hipError_t e2 = hipEventDestroy(t->stop);
+  delete t;
+  return (int)(e1 != hipSuccess ? e1 : e2);
+}
+int w2v_timer_start(void* timer) {
+  if (!timer) return (int)hipErrorInvalidValue;
+  return (int)hipEventRecord(static_cast<Timer*>(timer)->start, t_state.stream);
+}
+int w2v_timer_stop(void* timer) {
+  if (!timer) return (int)hipErrorInvalidValue;
+  return (int)hipEventRecord(static_cast<Timer*>(timer)->stop, t_state.stream);
+}
+int w2v_timer_elapsed_ms(void* timer, float* ms) {
+  if (!timer || !ms) return (int)hipErrorInvalidValue;
+  Timer* t = static_cast<Timer*>(timer);
+  hipError_t err = hipEventSynchronize(t->stop);
+  if (err != hipSuccess) return (int)err;
+  return (int)hipEventElapsedTime(ms, t->start, t->stop);
+}
+
+const char* w2v_error_string(int err) { return hipGetErrorString((hipError_t)err); }
+
+}  // extern "C"

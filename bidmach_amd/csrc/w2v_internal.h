@@ -1,0 +1,48 @@
+// Host-side declarations shared between the launchers and the C-ABI file.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Dispatch on R = ceil(nrows / 64), the registers per lane that hold one column.
+#define W2V_ROUNDS_SWITCH(R_, CALL)                                                        \
+  switch (R_) {                                                                            \
+    case 1: CALL(1); case 2: CALL(2); case 3: CALL(3); case 4: CALL(4); case 5: CALL(5);   \
+    case 6: CALL(6); case 7: CALL(7); case 8: CALL(8); case 9: CALL(9); case 10: CALL(10); \
+    case 11: CALL(11); case 12: CALL(12); case 13: CALL(13); case 14: CALL(14);            \
+    case 15: CALL(15); case 16: CALL(16); case 17: CALL(17); case 18: CALL(18);            \
+    case 19: CALL(19); case 20: CALL(20);                                                  \
+    default: return hipErrorInvalidValue;                                                  \
+  }
+
+namespace w2v {
+
+// Number of per-block partial sums an Eval launch over `units` work units writes.
+int64_t eval_partials_needed(int64_t units);
+
+// All launchers enqueue on `stream` and return the launch status; none of them synchronises.
+hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                      const int* UB, float* A, float* B, float lrate, float vexp);
+
+hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
+                      const int* WB, float* A, float* B, float lrate, float vexp);
+
+// Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
+// and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or
+// Retval64[0] (double, added into).  Either output pointer may be null.
+hipError_t launch_eval_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                           const int* UB, const float* A, const float* B, double floorv,
+                           double* partials, float* Retval32, double* Retval64);
+
+hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                           const int* WA, const int* WB, const float* A, const float* B,
+                           double floorv, double* partials, float* Retval32, double* Retval64);
+
+hipError_t launch_finalize(hipStream_t stream, const double* partials, int64_t n, float* Retval32,
+                           double* Retval64);
+
+// Largest nrows / nwb the register-resident kernels take; beyond them the calls fail with
+// hipErrorInvalidValue.
+int max_rows();
+int max_nwb();
+
+}  // namespace w2v

@@ -1,0 +1,196 @@
+// Negative-sample pass of skip-gram negative sampling, and its forward-only twin.
+//
+// Semantics follow the reference CPU path, jni/src/BIDMach_CPUMACH.c:186-264 (word2vecNeg) and
+// :429-483 (word2vecEvalNeg): group i holds nwa words WA[i*nwa + j] (columns of A) and nwb words
+// WB[i*nwb + k] (columns of B); for every (j, k):
+//   s = A[:,wa_j] . B[:,wb_k];  g = -lrate * sigmoid(s)
+//   dB_k += bscale_k * g * A[:,wa_j];   dA_j += ascale_j * g * B[:,wb_k]
+// and every dot product of the group uses the columns as they were when the group started; the
+// nwa + nwb accumulated deltas are scattered once each.
+//
+// One wavefront owns one group.  The nwb B columns and their nwb accumulators stay in registers;
+// A columns stream through CHA at a time (all loads of a chunk issued before its first dot).
+// The CHA*nwb pre-activations of a chunk are parked one per lane so that the sigmoid (a double
+// exp) is evaluated once per chunk; each A delta leaves as float atomics right after its chunk
+// and the B deltas after the last chunk, so every column is read once and updated once per
+// group.
+//
+// The reference reads WA/WB without a validity test (:213-214,220-221); here a negative id
+// skips every pair it takes part in, so a bad id cannot become an out-of-bounds access.
+#include "w2v_device.h"
+#include "w2v_internal.h"
+
+namespace w2v {
+
+template <int R, int MAXB, int CHA, bool TRAIN>
+__global__ void __launch_bounds__(kBlock)
+neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __restrict__ WA,
+           const int* __restrict__ WB, float* A, float* B, float lrate, float vexp, int smode,
+           double floorv, double* __restrict__ partials) {
+  static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t unit = xcd_contiguous_block(per_xcd) * kWavesPerBlock + wave;
+  double lsum = 0.0;
+
+  if (unit < ngroups) {
+    // Lane k < nwb holds B word k and its scale.
+    int wbl = -1;
+    if (lane < nwb) wbl = WB[unit * nwb + lane];
+    const float sbl = (TRAIN && wbl >= 0) ? scale_of(wbl, vexp, smode) : 0.0f;
+
+    float b[MAXB][R];
+    float dbb[MAXB][R];
+    int wb[MAXB];
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      wb[k] = -1;
+      if (k < nwb) {
+        wb[k] = read_lane(wbl, k);
+        if (wb[k] >= 0) load_col<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
+        if (TRAIN) zero_col<R>(dbb[k]);
+      }
+    }
+
+    for (int jbase = 0; jbase < nwa; jbase += kWave) {
+      // Lane l holds A word jbase+l and its scale.
+      int wal = -1;
+      if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
+      const float sal = (TRAIN && wal >= 0) ? scale_of(wal, vexp, smode) : 0.0f;
+      const int jend = min(nwa - jbase, kWave);
+
+      for (int j0 = 0; j0 < jend; j0 += CHA) {
+        float a[CHA][R];
+        int wa[CHA];
+#pragma unroll
+        for (int c = 0; c < CHA; ++c) {
+          wa[c] = -1;
+          if (j0 + c < jend) {
+            wa[c] = read_lane(wal, j0 + c);
+            if (wa[c] >= 0) load_col<R>(a[c], A + (int64_t)wa[c] * d, lane, d);
+          }
+        }
+        // Pre-activation of (c, k) parks in lane c*MAXB + k; lanes without a valid pair keep a
+        // marker below the lower clamp and are masked out afterwards.
+        float pre = 0.0f;
+        bool live = false;
+#pragma unroll
+        for (int c = 0; c < CHA; ++c) {
+          if (wa[c] >= 0) {
+#pragma unroll
+            for (int k = 0; k < MAXB; ++k) {
+              if (wb[k] >= 0) {
+                const float s = wave_sum(dot_partial<R>(a[c], b[k]));
+                const bool mine = lane == c * MAXB + k;
+                pre = mine ? s : pre;
+                live = mine ? true : live;
+              }
+            }
+          }
+        }
+        const float sg = sat_sigmoid(pre);
+        if (TRAIN) {
+          const float gl = -lrate * sg;
+#pragma unroll
+          for (int c = 0; c < CHA; ++c) {
+            if (wa[c] >= 0) {
+              const float as = read_lane(sal, j0 + c);
+              float daa[R];
+              zero_col<R>(daa);
+#pragma unroll
+              for (int k = 0; k < MAXB; ++k) {
+                if (wb[k] >= 0) {
+                  const float g = read_lane(gl, c * MAXB + k);
+                  const float bs = read_lane(sbl, k);
+                  axpy<R>(dbb[k], bs * g, a[c]);
+                  axpy<R>(daa, as * g, b[k]);
+                }
+              }
+              atomic_add_col<R>(A + (int64_t)wa[c] * d, daa, lane, d);
+            }
+          }
+        } else {
+          if (live) lsum += log(fmax(1.0 - (double)sg, floorv));
+        }
+      }
+    }
+
+    if (TRAIN) {
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k) {
+        if (wb[k] >= 0) atomic_add_col<R>(B + (int64_t)wb[k] * d, dbb[k], lane, d);
+      }
+    }
+  }
+
+  if (!TRAIN) {
+    const double wsum = wave_sum_f64(lsum);
+    block_store_partial(wsum, partials);
+  }
+}
+
+constexpr int kMaxNwb = 8;
+int max_nwb() { return kMaxNwb; }
+
+// A columns gathered per chunk, sized so that b, dbb and the chunk stay near 128 registers.
+template <int R, int MAXB>
+struct NegChunk {
+  static constexpr int budget = (128 - 2 * MAXB * R) / R;
+  static constexpr int capped = budget > 8 ? 8 : budget;
+  static constexpr int value = capped < 1 ? 1 : capped;
+};
+
+template <int R, int MAXB, bool TRAIN>
+static hipError_t launch_neg_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
+                                const int* WA, const int* WB, float* A, float* B, float lrate,
+                                float vexp, double floorv, double* partials) {
+  const int64_t per_xcd = blocks_per_xcd(ngroups);
+  const dim3 grid((unsigned)(per_xcd * kXcds));
+  hipLaunchKernelGGL((neg_kernel<R, MAXB, NegChunk<R, MAXB>::value, TRAIN>), grid, dim3(kBlock), 0,
+                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, lrate, vexp,
+                     scale_mode(vexp), floorv, partials);
+  return hipGetLastError();
+}
+
+template <int R, bool TRAIN>
+static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
+                               const int* WA, const int* WB, float* A, float* B, float lrate,
+                               float vexp, double floorv, double* partials) {
+  if (nwb <= 2)
+    return launch_neg_rb<R, 2, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, vexp,
+                                      floorv, partials);
+  if (nwb <= 5)
+    return launch_neg_rb<R, 5, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, vexp,
+                                      floorv, partials);
+  if (nwb <= kMaxNwb)
+    return launch_neg_rb<R, kMaxNwb, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate,
+                                            vexp, floorv, partials);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
+                      const int* WB, float* A, float* B, float lrate, float vexp) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+#define CALL(R)                                                                                   \
+  return launch_neg_r<R, true>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, 0.0,    \
+                               nullptr)
+  W2V_ROUNDS_SWITCH(rounds, CALL)
+#undef CALL
+}
+
+hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                           const int* WA, const int* WB, const float* A, const float* B,
+                           double floorv, double* partials, float* Retval32, double* Retval64) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+  hipError_t err = hipSuccess;
+#define CALL(R)                                                                                   \
+  err = launch_neg_r<R, false>(stream, nrows, ncols, nwa, nwb, WA, WB, const_cast<float*>(A),     \
+                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials);              \
+  break
+  W2V_ROUNDS_SWITCH(rounds, CALL)
+#undef CALL
+  if (err != hipSuccess) return err;
+  return launch_finalize(stream, partials, eval_partials_needed(ncols), Retval32, Retval64);
+}
+
+}  // namespace w2v

@@ -1,0 +1,115 @@
+/*
+ * C ABI of the MI355X (gfx950) skip-gram negative-sampling library.
+ *
+ * The first four functions are the drop-in boundary: they have the parameter lists of the
+ * reference's GPU operator launchers (jni/include/MatKernel.hpp:77,79,83,85), which its JNI glue
+ * (jni/src/BIDMach_CUMACH.cpp:434-493) calls on behalf of edu.berkeley.bid.CUMACH
+ * (src/main/java/edu/berkeley/bid/CUMACH.java:90,92,96,98).  Every pointer is a device pointer
+ * owned by the caller; the library never allocates, frees or keeps them.
+ *
+ * Layout: A and B are nrows x vocab, column-major, fp32: word w's vector is the contiguous run
+ * [w*nrows, (w+1)*nrows).  Word ids are int32.
+ *
+ * Error convention (reference: jni/src/DNN127.cu:1417-1419): 0 on success, otherwise the
+ * hipError_t value.  A shape or argument the library rejects returns hipErrorInvalidValue (1),
+ * as the reference's launchers return 1 for a shape they have no kernel for
+ * (DNN127.cu:1397,1414-1415,1435).  The library never aborts the process.
+ *
+ * Threading (reference: MatKernel.hpp:2 and the per-thread default stream of its build): the
+ * four reference calls block until the work is done.  Each host thread has its own launch stream
+ * (the null stream until w2v_set_stream is called) and its own Eval scratch buffer.
+ */
+#ifndef BIDMACH_W2V_H_
+#define BIDMACH_W2V_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- The reference operator API -------------------------------------------------------- */
+
+/* Replaces word2vecPos, MatKernel.hpp:77 / DNN127.cu:1389-1420; arithmetic of
+ * BIDMach_CPUMACH.c:10-78.  ncols tokens; token i with W[i] >= 0 is a centre word whose window
+ * is the offsets j in [LB[i], UB[i]], j != 0, 0 <= i+j < ncols, W[i+j] >= 0.  A is indexed by the
+ * centre word, B by the context word; both are updated in place.  `shift` (the reference's
+ * template selector, the maximum window half-width) is accepted and not needed: any window
+ * width works. */
+int word2vecPos(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A, float *B,
+                float lrate, float vexp);
+
+/* Replaces word2vecNeg, MatKernel.hpp:79 / DNN127.cu:1423-1452; arithmetic of
+ * BIDMach_CPUMACH.c:186-264.  ncols groups; group i pairs the nwa words WA[i*nwa + j] (columns of
+ * A) with the nwb words WB[i*nwb + k] (columns of B).  nwb <= w2v_max_nwb(). */
+int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A, float *B,
+                float lrate, float vexp);
+
+/* Replaces word2vecEvalPos, MatKernel.hpp:83 / DNN127.cu:1485-1516; arithmetic of
+ * BIDMach_CPUMACH.c:368-427.  Adds sum(log(max(sigmoid(a.b), floor))) over the valid pairs into
+ * the device float Retval[0] (the caller clears it first, Word2Vec.scala:476). */
+int word2vecEvalPos(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A, float *B,
+                    float *Retval);
+
+/* Replaces word2vecEvalNeg, MatKernel.hpp:85 / DNN127.cu:1519-1548; arithmetic of
+ * BIDMach_CPUMACH.c:429-483.  Adds sum(log(max(1 - sigmoid(a.b), floor))) into Retval[0]. */
+int word2vecEvalNeg(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A, float *B,
+                    float *Retval);
+
+/* ---- Extensions with no counterpart in the reference's GPU API ------------------------- */
+
+/* Same sums, added into a device double (the reference's CPU twins return jdouble,
+ * BIDMach_CPUMACH.c:368,429; its GPU path keeps only a float). */
+int word2vecEvalPosF64(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A,
+                       float *B, double *Retval);
+int word2vecEvalNegF64(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
+                       float *B, double *Retval);
+
+/* Enqueue-only forms of the four operators: same arguments, same results, but they return after
+ * the launch; completion is observed with w2v_synchronize() or a timer. */
+int word2vecPosAsync(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A, float *B,
+                     float lrate, float vexp);
+int word2vecNegAsync(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A, float *B,
+                     float lrate, float vexp);
+int word2vecEvalPosAsync(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A,
+                         float *B, float *Retval);
+int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
+                         float *B, float *Retval);
+
+/* Floor inside the Eval logarithms, process-wide.  Default 1e-40 (BIDMach_CPUMACH.c:409,467);
+ * the reference's Scala and CUDA twins use 1e-20 (Word2Vec.scala:995,1123; DNN127.cu:310,916). */
+void w2v_set_eval_floor(double floor_value);
+double w2v_get_eval_floor(void);
+
+/* Launch stream of the calling thread (a hipStream_t passed as void*; NULL = the null stream). */
+int w2v_set_stream(void *stream);
+void *w2v_get_stream(void);
+int w2v_synchronize(void);
+
+/* Limits of the kernels: largest nrows and largest nwb. */
+int w2v_max_rows(void);
+int w2v_max_nwb(void);
+
+/* Device buffers for hosts that have no HIP binding of their own (the reference's host owns its
+ * buffers through JCuda; Word2Vec.scala:373 passes their raw pointers). */
+int w2v_malloc(void **dev_ptr, size_t bytes);
+int w2v_free(void *dev_ptr);
+int w2v_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes);
+int w2v_memcpy_d2h(void *host_dst, const void *dev_src, size_t bytes);
+int w2v_memset(void *dev_ptr, int value, size_t bytes);
+
+/* Event-pair timers on the calling thread's launch stream. */
+int w2v_timer_create(void **timer);
+int w2v_timer_destroy(void *timer);
+int w2v_timer_start(void *timer);
+int w2v_timer_stop(void *timer);
+int w2v_timer_elapsed_ms(void *timer, float *ms); /* waits for the stop event */
+
+/* Text of an error code returned by any function above. */
+const char *w2v_error_string(int err);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* BIDMACH_W2V_H_ */

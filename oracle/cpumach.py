@@ -1,0 +1,92 @@
+"""ctypes binding of the C oracle, shaped like the reference's CPU operator class.
+
+TEST INFRASTRUCTURE: only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg
+import this module.  The method names and argument lists are those of
+src/main/java/edu/berkeley/bid/CPUMACH.java:12,17,26,28 of the reference (numpy arrays stand
+in for Java primitive arrays; A and B are updated in place).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libw2v_oracle.so")
+_lib = None
+
+C_FLOOR = 1.0e-40      # jni/src/BIDMach_CPUMACH.c:409,467
+SCALA_FLOOR = 1.0e-20  # Word2Vec.scala:995,1123 and DNN127.cu:310,916
+
+
+def build(force=False):
+    """Compile the oracle with the reference's CPU flags (oracle/Makefile)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    ip = ctypes.POINTER(ctypes.c_int)
+    fp = ctypes.POINTER(ctypes.c_float)
+    ci, cf, cd = ctypes.c_int, ctypes.c_float, ctypes.c_double
+    lib.oracle_word2vecPos.argtypes = [ci, ci, ci, ip, ip, ip, fp, fp, cf, cf, ci]
+    lib.oracle_word2vecPos.restype = None
+    lib.oracle_word2vecNeg.argtypes = [ci, ci, ci, ci, ip, ip, fp, fp, cf, cf, ci]
+    lib.oracle_word2vecNeg.restype = None
+    lib.oracle_word2vecEvalPos.argtypes = [ci, ci, ci, ip, ip, ip, fp, fp, cd, ci]
+    lib.oracle_word2vecEvalPos.restype = cd
+    lib.oracle_word2vecEvalNeg.argtypes = [ci, ci, ci, ci, ip, ip, fp, fp, cd, ci]
+    lib.oracle_word2vecEvalNeg.restype = cd
+    lib.oracle_max_threads.restype = ci
+    _lib = lib
+    return lib
+
+
+def _i(a):
+    assert a.dtype == np.int32 and (a.flags.c_contiguous or a.flags.f_contiguous)
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+
+
+def _f(a):
+    assert a.dtype == np.float32 and (a.flags.c_contiguous or a.flags.f_contiguous)
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def max_threads():
+    return int(_load().oracle_max_threads())
+
+
+class CPUMACH:
+    """Same static-method surface as edu.berkeley.bid.CPUMACH for the four SGNS calls.
+
+    Model matrices are nrows x vocab, column-major: pass numpy arrays of shape (vocab, nrows)
+    in C order (word w's vector is row w), which is the same memory layout.
+    """
+
+    @staticmethod
+    def word2vecPos(nrows, ncols, skip, W, LB, UB, A, B, lrate, vexp, nthreads):
+        _load().oracle_word2vecPos(nrows, ncols, skip, _i(W), _i(LB), _i(UB), _f(A), _f(B),
+                                   lrate, vexp, nthreads)
+
+    @staticmethod
+    def word2vecNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, nthreads):
+        _load().oracle_word2vecNeg(nrows, ncols, nwa, nwb, _i(WA), _i(WB), _f(A), _f(B),
+                                   lrate, vexp, nthreads)
+
+    @staticmethod
+    def word2vecEvalPos(nrows, ncols, skip, W, LB, UB, A, B, nthreads, floor=C_FLOOR):
+        return float(_load().oracle_word2vecEvalPos(nrows, ncols, skip, _i(W), _i(LB), _i(UB),
+                                                    _f(A), _f(B), floor, nthreads))
+
+    @staticmethod
+    def word2vecEvalNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, nthreads, floor=C_FLOOR):
+        return float(_load().oracle_word2vecEvalNeg(nrows, ncols, nwa, nwb, _i(WA), _i(WB),
+                                                    _f(A), _f(B), floor, nthreads))

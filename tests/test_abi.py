@@ -1,0 +1,62 @@
+"""The C-ABI library loads and exports every function include/bidmach_w2v.h declares (no GPU)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from bidmach_amd import cumach
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bidmach_w2v.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//.*", "", text)
+    return sorted(set(re.findall(r"\b(word2vec\w+|w2v_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_four_reference_entry_points():
+    names = declared_functions()
+    for n in ("word2vecPos", "word2vecNeg", "word2vecEvalPos", "word2vecEvalNeg"):
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(cumach.lib_path()):
+        pytest.fail("HIP library not built: run `python -m bidmach_amd.build`")
+    lib = cumach.load_library()
+    names = declared_functions()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), n
+    out = subprocess.check_output(["nm", "-D", "--defined-only", cumach.lib_path()], text=True)
+    exported = set(line.split()[-1] for line in out.splitlines() if " T " in line)
+    for n in names:
+        assert n in exported, n
+
+
+def test_python_binding_covers_the_header():
+    assert sorted(cumach.SYMBOLS) == declared_functions()
+
+
+def test_header_compiles_as_c():
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c",
+                           HEADER])
+
+
+def test_limits_and_floor_without_gpu():
+    lib = cumach.load_library()
+    assert lib.w2v_max_rows() == 1280
+    assert lib.w2v_max_nwb() == 8
+    assert lib.w2v_get_eval_floor() == 1.0e-40
+    lib.w2v_set_eval_floor(1.0e-20)
+    assert lib.w2v_get_eval_floor() == 1.0e-20
+    lib.w2v_set_eval_floor(1.0e-40)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(cumach.W2VLibraryError):
+        cumach.load_library(str(tmp_path / "nope.so"))

@@ -1,0 +1,329 @@
+"""Parity of the HIP operators with the CPU oracle, called through the C ABI (needs an MI355X).
+
+Tolerances are the ones the task states: Eval sums within 1e-5 relative; updates within 1e-4
+absolute per element on collision-free minibatches.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from bidmach_amd import corpus
+
+pytestmark = pytest.mark.gpu
+
+EVAL_RTOL = 1e-5
+UPDATE_ATOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from bidmach_amd.cumach import CUMACH, load_library
+    load_library()
+    return torch, CUMACH
+
+
+def dev(torch, x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def rand_tables(rng, vocab, d, scale=0.3):
+    A = (rng.standard_normal((vocab, d)) * scale).astype(np.float32)
+    B = (rng.standard_normal((vocab, d)) * scale).astype(np.float32)
+    return A, B
+
+
+def gpu_eval_pos(gpu, d, skip, W, LB, UB, A, B, f64=False):
+    torch, CUMACH = gpu
+    ret = torch.zeros(1, dtype=torch.float64 if f64 else torch.float32, device="cuda")
+    fn = CUMACH.word2vecEvalPosF64 if f64 else CUMACH.word2vecEvalPos
+    err = fn(d, W.shape[0], skip, dev(torch, W), dev(torch, LB), dev(torch, UB), dev(torch, A),
+             dev(torch, B), ret)
+    assert err == 0
+    return float(ret.item())
+
+
+def gpu_eval_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, f64=False):
+    torch, CUMACH = gpu
+    ret = torch.zeros(1, dtype=torch.float64 if f64 else torch.float32, device="cuda")
+    fn = CUMACH.word2vecEvalNegF64 if f64 else CUMACH.word2vecEvalNeg
+    err = fn(d, G, nwa, nwb, dev(torch, WA), dev(torch, WB), dev(torch, A), dev(torch, B), ret)
+    assert err == 0
+    return float(ret.item())
+
+
+def gpu_pos(gpu, d, skip, W, LB, UB, A, B, lr, vexp):
+    torch, CUMACH = gpu
+    Ad, Bd = dev(torch, A), dev(torch, B)
+    err = CUMACH.word2vecPos(d, W.shape[0], skip, dev(torch, W), dev(torch, LB), dev(torch, UB),
+                             Ad, Bd, lr, vexp)
+    assert err == 0
+    return Ad.cpu().numpy(), Bd.cpu().numpy()
+
+
+def gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, lr, vexp):
+    torch, CUMACH = gpu
+    Ad, Bd = dev(torch, A), dev(torch, B)
+    err = CUMACH.word2vecNeg(d, G, nwa, nwb, dev(torch, WA), dev(torch, WB), Ad, Bd, lr, vexp)
+    assert err == 0
+    return Ad.cpu().numpy(), Bd.cpu().numpy()
+
+
+# ---------------------------------------------------------------------------------------------
+# Eval (forward only)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("d,V,N,skip", [
+    (100, 1000, 20000, 5), (300, 5000, 30000, 5), (512, 2000, 8000, 10), (1, 10, 100, 2),
+    (64, 300, 3000, 3), (65, 300, 3000, 3), (1280, 200, 500, 5), (37, 100, 2000, 40),
+])
+def test_eval_pos_matches_oracle(gpu, oracle, d, V, N, skip):
+    rng = np.random.default_rng(d + N)
+    A, B = rand_tables(rng, V, d, 0.6 / math.sqrt(d) ** 0.5)
+    W = corpus.zipf_stream(N, V, 1.0, seed=d)
+    W[rng.random(N) < 0.07] = -1
+    sent = np.cumsum(rng.random(N) < 0.03)
+    LB, UB = corpus.window_bounds(N, skip, rng, sentence=sent)
+    want = oracle.word2vecEvalPos(d, N, skip, W, LB, UB, A, B, 4)
+    assert want < -1.0
+    got32 = gpu_eval_pos(gpu, d, skip, W, LB, UB, A, B)
+    got64 = gpu_eval_pos(gpu, d, skip, W, LB, UB, A, B, f64=True)
+    assert got64 == pytest.approx(want, rel=EVAL_RTOL)
+    assert got32 == pytest.approx(want, rel=EVAL_RTOL)
+
+
+@pytest.mark.parametrize("d,V,G,nwa,nwb", [
+    (100, 1000, 5000, 5, 5), (300, 5000, 6000, 5, 5), (512, 2000, 2000, 15, 5), (1, 10, 50, 1, 1),
+    (64, 300, 500, 3, 2), (65, 300, 500, 7, 8), (1280, 200, 100, 5, 5), (50, 400, 300, 70, 4),
+    (300, 500, 1000, 9, 1),
+])
+def test_eval_neg_matches_oracle(gpu, oracle, d, V, G, nwa, nwb):
+    rng = np.random.default_rng(d + G)
+    A, B = rand_tables(rng, V, d, 0.6 / math.sqrt(d) ** 0.5)
+    WA = rng.integers(0, V, G * nwa).astype(np.int32)
+    WB = corpus.zipf_stream(G * nwb, V, 1.0, seed=G)
+    want = oracle.word2vecEvalNeg(d, G, nwa, nwb, WA, WB, A, B, 4)
+    got32 = gpu_eval_neg(gpu, d, G, nwa, nwb, WA, WB, A, B)
+    got64 = gpu_eval_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, f64=True)
+    assert got64 == pytest.approx(want, rel=EVAL_RTOL)
+    assert got32 == pytest.approx(want, rel=EVAL_RTOL)
+
+
+def test_eval_is_deterministic_and_adds_into_retval(gpu, oracle):
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(1)
+    d, V, N = 300, 3000, 50000
+    A, B = rand_tables(rng, V, d, 0.1)
+    W = corpus.zipf_stream(N, V, 1.0, seed=3)
+    LB, UB = corpus.window_bounds(N, 5, rng)
+    a = gpu_eval_pos(gpu, d, 5, W, LB, UB, A, B, f64=True)
+    b = gpu_eval_pos(gpu, d, 5, W, LB, UB, A, B, f64=True)
+    assert a == b
+    # the float result is added into Retval[0], as the reference kernel does (DNN127.cu:322-324)
+    ret = torch.full((1,), 1000.0, dtype=torch.float32, device="cuda")
+    err = CUMACH.word2vecEvalPos(d, N, 5, dev(torch, W), dev(torch, LB), dev(torch, UB),
+                                 dev(torch, A), dev(torch, B), ret)
+    assert err == 0
+    assert float(ret.item()) == pytest.approx(1000.0 + a, rel=1e-6)
+
+
+@pytest.mark.parametrize("s,pos_want,neg_want,neg_abs", [
+    (16.5, 0.0, math.log(1e-40), 1e-9),
+    (-16.5, math.log(1e-40), 0.0, 1e-9),
+    (16.0, -math.log1p(math.exp(-16.0)), -16.0, 0.1),
+    (-16.0, -16.0 - math.log1p(math.exp(-16.0)), -math.log1p(math.exp(-16.0)), 2e-7),
+])
+def test_clamps_and_floor_on_gpu(gpu, oracle, s, pos_want, neg_want, neg_abs):
+    A = np.array([[1.0], [0.0]], np.float32)
+    B = np.array([[0.0], [s]], np.float32)
+    W = np.array([0, 1], np.int32)
+    LB = np.array([0, 0], np.int32)
+    UB = np.array([1, 0], np.int32)
+    got = gpu_eval_pos(gpu, 1, 1, W, LB, UB, A, B, f64=True)
+    assert got == pytest.approx(pos_want, rel=1e-6, abs=2e-7)
+    assert got == pytest.approx(oracle.word2vecEvalPos(1, 2, 1, W, LB, UB, A, B, 1), rel=1e-6,
+                                abs=1e-12)
+    WA = np.array([0], np.int32)
+    WB = np.array([1], np.int32)
+    got = gpu_eval_neg(gpu, 1, 1, 1, 1, WA, WB, A, B, f64=True)
+    assert got == pytest.approx(neg_want, rel=1e-6, abs=neg_abs)
+    assert got == pytest.approx(oracle.word2vecEvalNeg(1, 1, 1, 1, WA, WB, A, B, 1), rel=1e-6,
+                                abs=1e-12)
+
+
+def test_eval_floor_switch(gpu):
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    A = np.array([[1.0], [0.0]], np.float32)
+    B = np.array([[0.0], [-20.0]], np.float32)
+    W = np.array([0, 1], np.int32)
+    LB = np.array([0, 0], np.int32)
+    UB = np.array([1, 0], np.int32)
+    try:
+        lib.w2v_set_eval_floor(1.0e-20)
+        assert gpu_eval_pos(gpu, 1, 1, W, LB, UB, A, B, f64=True) == \
+            pytest.approx(math.log(1e-20), rel=1e-12)
+    finally:
+        lib.w2v_set_eval_floor(1.0e-40)
+    assert gpu_eval_pos(gpu, 1, 1, W, LB, UB, A, B, f64=True) == \
+        pytest.approx(math.log(1e-40), rel=1e-12)
+
+
+# ---------------------------------------------------------------------------------------------
+# Updates on collision-free minibatches
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("vexp", [0.0, 0.5, 1.0, 0.75])
+@pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (512, 10, 100),
+                                             (1, 2, 50), (65, 3, 100), (1280, 5, 40),
+                                             (24, 40, 30)])
+def test_pos_update_matches_oracle(gpu, oracle, vexp, d, skip, ncentres):
+    rng = np.random.default_rng(d * 7 + skip)
+    V = 20000
+    A, B = rand_tables(rng, V, d, 0.5 / math.sqrt(d) ** 0.5)
+    W, LB, UB = corpus.collision_free_pos(ncentres, skip, V, rng)
+    W[rng.random(W.shape[0]) < 0.05] = -1
+    lr = 0.025 if vexp < 1.0 else 0.001
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecPos(d, W.shape[0], skip, W, LB, UB, Ao, Bo, lr, vexp, 1)
+    Ag, Bg = gpu_pos(gpu, d, skip, W, LB, UB, A, B, lr, vexp)
+    assert np.abs(Ag - Ao).max() <= UPDATE_ATOL
+    assert np.abs(Bg - Bo).max() <= UPDATE_ATOL
+    assert np.abs(Ao - A).max() > 10 * UPDATE_ATOL or d == 1
+
+
+@pytest.mark.parametrize("vexp", [0.0, 0.5, 1.0, 0.75])
+@pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
+                                         (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
+                                         (40, 70, 3, 40), (300, 6, 2, 100)])
+def test_neg_update_matches_oracle(gpu, oracle, vexp, d, nwa, nwb, G):
+    rng = np.random.default_rng(d * 5 + nwa)
+    V = 20000
+    A, B = rand_tables(rng, V, d, 0.5 / math.sqrt(d) ** 0.5)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    lr = 0.025 if vexp < 1.0 else 0.001
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, lr, vexp, 1)
+    Ag, Bg = gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, lr, vexp)
+    assert np.abs(Ag - Ao).max() <= UPDATE_ATOL
+    assert np.abs(Bg - Bo).max() <= UPDATE_ATOL
+    assert np.abs(Ao - A).max() > 10 * UPDATE_ATOL or d == 1
+
+
+def test_noop_invariants_on_gpu(gpu):
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(6)
+    d, V, N = 300, 500, 3000
+    A, B = rand_tables(rng, V, d)
+    W = rng.integers(0, V, N).astype(np.int32)
+    LB, UB = corpus.window_bounds(N, 5, rng)
+    WA = rng.integers(0, V, 500).astype(np.int32)
+    WB = rng.integers(0, V, 500).astype(np.int32)
+    Ag, Bg = gpu_pos(gpu, d, 5, W, LB, UB, A, B, 0.0, 0.5)
+    assert np.array_equal(Ag, A) and np.array_equal(Bg, B)
+    Ag, Bg = gpu_neg(gpu, d, 100, 5, 5, WA, WB, A, B, 0.0, 0.5)
+    assert np.array_equal(Ag, A) and np.array_equal(Bg, B)
+    Ag, Bg = gpu_pos(gpu, d, 5, np.full(N, -1, np.int32), LB, UB, A, B, 0.1, 0.5)
+    assert np.array_equal(Ag, A) and np.array_equal(Bg, B)
+    Z = np.zeros(N, np.int32)
+    Ag, Bg = gpu_pos(gpu, d, 5, W, Z, Z, A, B, 0.1, 0.5)
+    assert np.array_equal(Ag, A) and np.array_equal(Bg, B)
+    assert gpu_eval_pos(gpu, d, 5, W, Z, Z, A, B) == 0.0
+
+
+def test_empty_and_rejected_arguments(gpu):
+    torch, CUMACH = gpu
+    d = 300
+    A = torch.zeros(10, d, device="cuda")
+    B = torch.zeros(10, d, device="cuda")
+    I = torch.zeros(16, dtype=torch.int32, device="cuda")
+    ret = torch.zeros(1, device="cuda")
+    # empty minibatch: success, nothing touched
+    assert CUMACH.word2vecPos(d, 0, 5, I, I, I, A, B, 0.1, 0.5) == 0
+    assert CUMACH.word2vecNeg(d, 0, 5, 5, I, I, A, B, 0.1, 0.5) == 0
+    assert CUMACH.word2vecEvalPos(d, 0, 5, I, I, I, A, B, ret) == 0
+    assert CUMACH.word2vecEvalNeg(d, 0, 5, 5, I, I, A, B, ret) == 0
+    assert float(ret.item()) == 0.0
+    # rejected shapes and null pointers: hipErrorInvalidValue (1), no launch, no abort
+    assert CUMACH.word2vecPos(0, 4, 5, I, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecPos(1281, 4, 5, I, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecPos(d, -1, 5, I, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecPos(d, 4, 5, None, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecNeg(d, 1, 5, 9, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecNeg(d, 1, 5, 5, I, None, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecEvalPos(d, 4, 5, I, I, I, A, B, None) == 1
+    assert CUMACH.word2vecEvalNeg(d, 1, 5, 5, I, I, A, None, ret) == 1
+    # the library is still usable afterwards
+    assert CUMACH.word2vecEvalPos(d, 4, 5, I, I, I, A, B, ret) == 0
+
+
+def test_negative_ids_in_groups_are_skipped(gpu, oracle):
+    """The reference reads WA/WB unchecked; the library skips pairs with a negative id."""
+    rng = np.random.default_rng(31)
+    d, V, G, nwa, nwb = 100, 5000, 60, 5, 5
+    A, B = rand_tables(rng, V, d, 0.3)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    WA2, WB2 = WA.copy(), WB.copy()
+    WA2[3] = -1
+    WB2[7] = -1
+    Ag, Bg = gpu_neg(gpu, d, G, nwa, nwb, WA2, WB2, A, B, 0.05, 0.5)
+    # expected: closed form with those pairs removed = oracle on groups rebuilt without them
+    from oracle import closed_form as cf
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    for g in range(G):
+        wa = [w for w in WA2[g * nwa:(g + 1) * nwa] if w >= 0]
+        wb = [w for w in WB2[g * nwb:(g + 1) * nwb] if w >= 0]
+        Aw, Bw = cf.neg_update(len(wa), len(wb), np.array(wa), np.array(wb), A, B, 0.05, 0.5)
+        for w in wa:
+            np.testing.assert_allclose(Ag[w], Aw[w], atol=UPDATE_ATOL, rtol=0)
+        for w in wb:
+            np.testing.assert_allclose(Bg[w], Bw[w], atol=UPDATE_ATOL, rtol=0)
+    assert np.array_equal(Ag[WA[3]], A[WA[3]])
+    assert np.array_equal(Bg[WB[7]], B[WB[7]])
+
+
+# ---------------------------------------------------------------------------------------------
+# Colliding (Zipf) minibatches: statistical agreement
+# ---------------------------------------------------------------------------------------------
+
+def _rows_close(got, want, rtol, atol):
+    err = np.abs(got - want).max(axis=1)
+    lim = rtol * np.abs(want).max(axis=1) + atol
+    bad = np.flatnonzero(err > lim)
+    assert bad.size == 0, (bad[:5], err[bad[:5]], lim[bad[:5]])
+
+
+def test_heavy_collisions_lose_no_contribution(gpu):
+    """With one table at zero every dot product is 0 and g = lr/2 (or -lr/2) whatever the order
+    of the Hogwild updates, so the result on a Zipf minibatch with thousands of collisions per
+    column is known exactly: the other table's delta is scale*g*sum(partner columns)."""
+    from oracle import closed_form as cf
+    rng = np.random.default_rng(41)
+    d, V, N, lr = 100, 300, 20000, 0.025
+    T = (rng.standard_normal((V, d)) * 0.2).astype(np.float32)
+    Z = np.zeros((V, d), np.float32)
+    W = corpus.zipf_stream(N, V, 1.0, seed=9)
+    W[rng.random(N) < 0.05] = -1
+    LB, UB = corpus.window_bounds(N, 5, rng)
+    WA, WB, G = corpus.negative_groups(W, LB, UB, 5, 5, rng, vocab=V)
+    for vexp in (0.0, 0.5):
+        # A = 0: only A moves (centre / negative side)
+        Ag, Bg = gpu_pos(gpu, d, 5, W, LB, UB, Z, T, lr, vexp)
+        Aw, Bw = cf.pos_update(W, LB, UB, Z, T, lr, vexp)
+        assert np.array_equal(Bg, T)
+        _rows_close(Ag, Aw, 2e-5, 1e-6)
+        Ag, Bg = gpu_neg(gpu, d, G, 5, 5, WA, WB, Z, T, lr, vexp)
+        Aw, Bw = cf.neg_update(5, 5, WA, WB, Z, T, lr, vexp)
+        assert np.array_equal(Bg, T)
+        _rows_close(Ag, Aw, 2e-5, 1e-6)
+        # B = 0: only B moves (context side)
+        Ag, Bg = gpu_pos(gpu, d, 5, W, LB, UB, T, Z, lr, vexp)
+        Aw, Bw = cf.pos_update(W, LB, UB, T, Z, lr, vexp)
+        assert np.array_equal(Ag, T)
+        _rows_close(Bg, Bw, 2e-5, 1e-6)
+        Ag, Bg = gpu_neg(gpu, d, G, 5, 5, WA, WB, T, Z, lr, vexp)
+        Aw, Bw = cf.neg_update(5, 5, WA, WB, T, Z, lr, vexp)
+        assert np.array_equal(Ag, T)
+        _rows_close(Bg, Bw, 2e-5, 1e-6)
