@@ -64,12 +64,12 @@ int finish(hipError_t launch_err, bool sync) {
   return 0;
 }
 
-int pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, float* B, float lrate,
-             float vexp, bool sync) {
+int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
+             float lrate, float vexp, bool sync) {
   if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp), sync);
+  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp), sync);
 }
 
 int neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
@@ -120,8 +120,7 @@ extern "C" {
 
 int word2vecPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
                 float lrate, float vexp) {
-  (void)shift;
-  return pos_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, true);
+  return pos_impl(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, true);
 }
 
 int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
@@ -153,8 +152,7 @@ int word2vecEvalNegF64(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
 
 int word2vecPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
                      float lrate, float vexp) {
-  (void)shift;
-  return pos_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, false);
+  return pos_impl(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, false);
 }
 
 int word2vecNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,

@@ -20,8 +20,10 @@ namespace w2v {
 int64_t eval_partials_needed(int64_t units);
 
 // All launchers enqueue on `stream` and return the launch status; none of them synchronises.
-hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                      const int* UB, float* A, float* B, float lrate, float vexp);
+// `shift` is the caller's maximum window half-width; it sizes the halo a tile stages in LDS.
+// Offsets beyond it are still processed (gathered from memory), so any LB/UB is accepted.
+hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp);
 
 hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
                       const int* WB, float* A, float* B, float lrate, float vexp);

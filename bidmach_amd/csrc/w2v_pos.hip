@@ -4,16 +4,32 @@
 // :368-427 (word2vecEvalPos): for each centre token i with W[i] >= 0 and each offset
 // j in [LB[i], UB[i]], j != 0, 0 <= i+j < ncols, W[i+j] >= 0:
 //   s = A[:,W[i]] . B[:,W[i+j]];  g = lrate * (1 - sigmoid(s))
-//   B[:,W[i+j]] += bscale * g * A[:,W[i]]      (scattered at once)
+//   B[:,W[i+j]] += bscale * g * A[:,W[i]]
 //   A[:,W[i]]   += ascale * g * B[:,W[i+j]]    (accumulated over the window, scattered once)
 //
-// One wavefront owns one centre token.  Its A column stays in registers for the whole window;
+// Two kernels.
+//
+// pos_kernel (forward-only scoring, and the update when a tile does not fit in LDS): one
+// wavefront owns one centre token.  Its A column stays in registers for the whole window;
 // context columns are gathered CH at a time (all loads of a chunk are issued before the first
 // dot product, so a wave keeps CH columns in flight), dot products are reduced with DPP row
-// rotations, the CH pre-activations are parked in lanes 0..CH-1 so that the sigmoid (a double
-// exp) is evaluated once per chunk instead of once per pair, and the updates leave as float
-// atomics.  A chunk reads its context columns before it updates any of them, so a word that
-// occurs twice inside one chunk sees the pre-chunk value (Hogwild staleness, as between waves).
+// rotations, and the CH pre-activations are parked in lanes 0..CH-1 so that the sigmoid (a double
+// exp) is evaluated once per chunk instead of once per pair.
+//
+// pos_tile_kernel (the update): float atomics are the scarce resource on this GPU (the L2
+// retires about one dword atomic per clock per channel, roughly 1.1 TB/s of payload for the
+// whole chip, whatever the footprint), so the update is organised to issue as few of them as
+// the data allows.  A workgroup owns a tile of T consecutive tokens.  It stages the A columns of
+// its T centres and the B columns of the T + 2*Sh positions its windows can reach in LDS
+// (each column is gathered from HBM once per tile instead of once per pair), then
+//   phase 1, one wave per centre: dot products against the staged B columns, sigmoid, the
+//     centre's delta accumulated in registers and scattered with one column of atomics; every
+//     g is left in an LDS table G[centre][offset];
+//   phase 2, one wave per staged position: the sum over the tile's centres of g * A column,
+//     scattered with one column of atomics.
+// A token therefore costs about (2T + 2Sh)/T columns of atomics instead of 1 + (pairs).
+// All dot products of a tile use the columns as staged (a tile is a small synchronous batch);
+// between tiles the updates are Hogwild, as between the reference's threads.
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
@@ -110,6 +126,160 @@ pos_kernel(int d, int ncols, int64_t per_xcd, const int* __restrict__ W,
   }
 }
 
+constexpr int kTileWaves = 8;
+constexpr int kTileThreads = kTileWaves * kWave;
+constexpr int kMaxHalo = 31;  // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
+
+// LDS layout of a tile: a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh]
+// with dp = R*64 (columns zero-padded so that LDS reads need no bounds test).
+__host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
+  const size_t dp = (size_t)R * kWave;
+  return ((size_t)T * dp + (size_t)(T + 2 * Sh) * dp + (size_t)T * (2 * Sh + 1) +
+          (size_t)(T + 2 * Sh)) * 4;
+}
+
+template <int R>
+__global__ void __launch_bounds__(kTileThreads)
+pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t per_xcd, const int* __restrict__ W,
+                const int* __restrict__ LB, const int* __restrict__ UB, float* A, float* B,
+                float lrate, float vexp, int smode) {
+  extern __shared__ float lds[];
+  constexpr int dp = R * kWave;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gw = 2 * Sh + 1;
+  float* const a_t = lds;
+  float* const b_t = a_t + (size_t)T * dp;
+  float* const G = b_t + (size_t)(T + 2 * Sh) * dp;
+  int* const wt = reinterpret_cast<int*>(G + (size_t)T * gw);
+
+  const int64_t tile = xcd_contiguous_block(per_xcd);
+  const int64_t lo64 = tile * T;
+  if (lo64 >= ncols) return;  // whole workgroup leaves together
+  const int lo = (int)lo64;
+  const int hi = min(lo + T, ncols);          // centres [lo, hi)
+  const int hlo = max(lo - Sh, 0);
+  const int hhi = min(hi + Sh, ncols);        // staged positions [hlo, hhi)
+  const int nh = hhi - hlo;
+  const int nc = hi - lo;
+
+  // ---- stage: word ids, B columns of every staged position, A columns of the centres ----
+  for (int c = wave; c < nh; c += kTileWaves) {
+    const int p = hlo + c;
+    const int w = W[p];
+    if (lane == 0) wt[c] = w;
+    if (w >= 0) {
+      float x[R];
+      load_col<R>(x, B + (int64_t)w * d, lane, d);
+#pragma unroll
+      for (int r = 0; r < R; ++r) b_t[(size_t)c * dp + r * kWave + lane] = x[r];
+      if (p >= lo && p < hi) {
+        load_col<R>(x, A + (int64_t)w * d, lane, d);
+#pragma unroll
+        for (int r = 0; r < R; ++r) a_t[(size_t)(p - lo) * dp + r * kWave + lane] = x[r];
+      }
+    }
+  }
+  for (int k = threadIdx.x; k < nc * gw; k += kTileThreads) G[k] = 0.0f;
+  __syncthreads();
+
+  // ---- phase 1: one wave per centre ----
+  for (int ci = wave; ci < nc; ci += kTileWaves) {
+    const int i = lo + ci;
+    const int wi = wt[i - hlo];
+    if (wi < 0) continue;
+    const int jlo = max(LB[i], -i);
+    const int jhi = min(UB[i], ncols - 1 - i);
+    float a[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) a[r] = a_t[(size_t)ci * dp + r * kWave + lane];
+    float daa[R];
+    zero_col<R>(daa);
+    const float ascale = scale_of(wi, vexp, smode);
+    bool touched = false;
+
+    // Staged part of the window: lane l stands for offset j = l - Sh.
+    {
+      const int j = lane - Sh;
+      const int c = i + j - hlo;  // staged slot of position i + j
+      int wl = -1;
+      if (lane < gw && j != 0 && j >= jlo && j <= jhi) wl = wt[c];
+      const unsigned long long valid = __ballot(wl >= 0);
+      if (valid != 0ull) {
+        float pre = 0.0f;
+        unsigned long long mask = valid;
+        while (mask != 0ull) {
+          const int l = __builtin_ctzll(mask);
+          mask &= mask - 1ull;
+          const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
+          float s = 0.0f;
+#pragma unroll
+          for (int r = 0; r < R; ++r) s = fmaf(a[r], bcol[r * kWave], s);
+          s = wave_sum(s);
+          pre = (lane == l) ? s : pre;
+        }
+        const float gl = lrate * (1.0f - sat_sigmoid(pre));
+        if (wl >= 0) G[ci * gw + lane] = gl;
+        mask = valid;
+        while (mask != 0ull) {
+          const int l = __builtin_ctzll(mask);
+          mask &= mask - 1ull;
+          const float ag = ascale * read_lane(gl, l);
+          const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
+#pragma unroll
+          for (int r = 0; r < R; ++r) daa[r] = fmaf(ag, bcol[r * kWave], daa[r]);
+        }
+        touched = true;
+      }
+    }
+
+    // Offsets beyond the staged halo (only when LB/UB exceed the caller's `shift`): one context
+    // at a time, gathered from memory and scattered at once.
+    for (int j = jlo; j <= jhi; ++j) {
+      if (j >= -Sh && j <= Sh) {
+        j = Sh;  // skip the staged range
+        continue;
+      }
+      const int wb = W[i + j];
+      if (wb < 0) continue;
+      float b[R];
+      load_col<R>(b, B + (int64_t)wb * d, lane, d);
+      const float s = wave_sum(dot_partial<R>(a, b));
+      const float g = lrate * (1.0f - sat_sigmoid(s));
+      axpy<R>(daa, ascale * g, b);
+      atomic_axpy_col<R>(B + (int64_t)wb * d, scale_of(wb, vexp, smode) * g, a, lane, d);
+      touched = true;
+    }
+    if (touched) atomic_add_col<R>(A + (int64_t)wi * d, daa, lane, d);
+  }
+  __syncthreads();
+
+  // ---- phase 2: one wave per staged position ----
+  for (int c = wave; c < nh; c += kTileWaves) {
+    const int wp = wt[c];
+    if (wp < 0) continue;
+    const int p = hlo + c;
+    // lane l looks at centre i = p - Sh + l; its g for this position sits at offset p - i
+    const int i = p - Sh + lane;
+    float gl = 0.0f;
+    if (lane < gw && i >= lo && i < hi && i != p) gl = G[(i - lo) * gw + (p - i + Sh)];
+    unsigned long long mask = __ballot(gl != 0.0f);
+    if (mask == 0ull) continue;
+    float dbb[R];
+    zero_col<R>(dbb);
+    while (mask != 0ull) {
+      const int l = __builtin_ctzll(mask);
+      mask &= mask - 1ull;
+      const float g = read_lane(gl, l);
+      const int ci = p - Sh + l - lo;
+#pragma unroll
+      for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, a_t[(size_t)ci * dp + r * kWave + lane], dbb[r]);
+    }
+    const float bs = scale_of(wp, vexp, smode);
+    atomic_axpy_col<R>(B + (int64_t)wp * d, bs, dbb, lane, d);
+  }
+}
+
 // Folds the per-block partial sums in a fixed order (thread t takes t, t+256, ...; then a
 // fixed LDS tree), so the result does not depend on block scheduling.
 __global__ void __launch_bounds__(kBlock)
@@ -151,11 +321,43 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
   return hipGetLastError();
 }
 
-hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                      const int* UB, float* A, float* B, float lrate, float vexp) {
+// Tile size: the largest power of two (8..64) whose LDS footprint lets three workgroups share a
+// CU; if even 8 tokens need more than one CU's LDS the per-centre kernel is used instead.
+static int pick_tile(int R, int Sh) {
+  constexpr size_t kShare = 52 * 1024, kLimit = 160 * 1024;
+  int T = 64;
+  while (T > 8 && tile_lds_bytes(R, T, Sh) > kShare) T >>= 1;
+  if (tile_lds_bytes(R, T, Sh) > kLimit) return 0;
+  return T;
+}
+
+template <int R>
+static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int shift, const int* W,
+                                    const int* LB, const int* UB, float* A, float* B, float lrate,
+                                    float vexp) {
+  const int Sh = shift < 0 ? 0 : (shift > kMaxHalo ? kMaxHalo : shift);
+  const int T = Sh > 0 ? pick_tile(R, Sh) : 0;
+  if (T == 0)
+    return launch_pos_r<R, true>(stream, d, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr);
+  const size_t lds = tile_lds_bytes(R, T, Sh);
+  auto kern = pos_tile_kernel<R>;
+  if (lds > 48 * 1024) {
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return err;
+  }
+  const int64_t ntiles = ((int64_t)ncols + T - 1) / T;
+  const int64_t per_xcd = (ntiles + kXcds - 1) / kXcds;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * kXcds)), dim3(kTileThreads), lds, stream, d,
+                     ncols, T, Sh, per_xcd, W, LB, UB, A, B, lrate, vexp, scale_mode(vexp));
+  return hipGetLastError();
+}
+
+hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp) {
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R) \
-  return launch_pos_r<R, true>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr)
+  return launch_pos_tile_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }
