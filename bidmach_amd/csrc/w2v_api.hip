@@ -15,6 +15,7 @@ struct ThreadState {
   hipStream_t stream = nullptr;
   double* partials[kMaxDevices] = {};
   int64_t capacity[kMaxDevices] = {};
+  float* shadow[kMaxDevices] = {};  // two shadow buffers (A then B), zero between calls
 };
 
 thread_local ThreadState t_state;
@@ -50,6 +51,30 @@ hipError_t eval_scratch(int64_t need, double** out) {
   return hipSuccess;
 }
 
+// Per-thread, per-device shadow buffers for the hot columns, allocated and zeroed on first use.
+hipError_t shadow_buffers(w2v::Shadow* out) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  ThreadState& ts = t_state;
+  const size_t bytes = w2v::shadow_bytes();
+  if (ts.shadow[dev] == nullptr) {
+    float* p = nullptr;
+    err = hipMalloc(reinterpret_cast<void**>(&p), 2 * bytes);
+    if (err != hipSuccess) return err;
+    err = hipMemsetAsync(p, 0, 2 * bytes, ts.stream);
+    if (err != hipSuccess) {
+      (void)hipFree(p);
+      return err;
+    }
+    ts.shadow[dev] = p;
+  }
+  out->a = ts.shadow[dev];
+  out->b = ts.shadow[dev] + bytes / sizeof(float);
+  return hipSuccess;
+}
+
 bool bad_common(int nrows, int ncols) {
   return nrows <= 0 || nrows > w2v::max_rows() || ncols < 0;
 }
@@ -69,7 +94,12 @@ int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A
   if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp), sync);
+  w2v::Shadow shadow{};
+  hipError_t err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp,
+                                shadow),
+                sync);
 }
 
 int neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
@@ -78,8 +108,12 @@ int neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A,
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
-  return finish(
-      w2v::launch_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp), sync);
+  w2v::Shadow shadow{};
+  hipError_t err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp,
+                                shadow),
+                sync);
 }
 
 int eval_pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, float* B, float* r32,

@@ -114,26 +114,82 @@ __device__ __forceinline__ void axpy(float (&y)[R], float alpha, const float (&x
   for (int r = 0; r < R; ++r) y[r] = fmaf(alpha, x[r], y[r]);
 }
 
-// Hogwild scatter: col[e] += alpha * x[e] with one hardware float atomic per lane and round
-// (global_atomic_add_f32, no return value, no compare-and-swap loop).
+// Hogwild scatter of a column held in the dword-strided register layout: col[e] += x[e] with
+// hardware float atomics (global_atomic_add_f32, no return value, no compare-and-swap loop).
+//
+// The L2 retires atomics per 128-byte line request, and a column starts wherever w*d*4 falls,
+// so a wave instruction that covers elements [64r, 64r+64) of the column straddles three lines.
+// The lanes are therefore rotated by the column's misalignment (ds_bpermute) so that every
+// instruction covers exactly two whole lines: lane l of round r' handles element
+// 64*r' + l - mis, where mis = (column start / 4) mod 32.  One extra, mostly empty, round pays
+// for roughly a third fewer line requests.
 template <int R>
-__device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float alpha,
-                                                const float (&x)[R], int lane, int d) {
+__device__ __forceinline__ void atomic_add_col(float* __restrict__ col, const float (&x)[R],
+                                               int lane, int d) {
+  const int mis = (int)((reinterpret_cast<uintptr_t>(col) >> 2) & 31u);
+  const int src = (lane - mis) & (kWave - 1);
+  float prev = 0.0f;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int e = r * kWave + lane;
-    if (r < R - 1 || e < d) unsafeAtomicAdd(col + e, alpha * x[r]);
+  for (int r = 0; r <= R; ++r) {
+    float cur = 0.0f;
+    if (r < R) cur = __shfl(x[r], src, kWave);
+    const float v = (lane >= mis) ? cur : prev;
+    const int e = r * kWave + lane - mis;
+    if (e >= 0 && e < d) unsafeAtomicAdd(col + e, v);
+    prev = cur;
   }
 }
 
 template <int R>
-__device__ __forceinline__ void atomic_add_col(float* __restrict__ col, const float (&x)[R],
-                                               int lane, int d) {
+__device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float alpha,
+                                                const float (&x)[R], int lane, int d) {
+  float y[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int e = r * kWave + lane;
-    if (r < R - 1 || e < d) unsafeAtomicAdd(col + e, x[r]);
+  for (int r = 0; r < R; ++r) y[r] = alpha * x[r];
+  atomic_add_col<R>(col, y, lane, d);
+}
+
+// Shadow copies of the hottest columns.
+//
+// Word ids are frequency ranks, so under a Zipf law ids 0..7 each receive hundreds of thousands
+// of column updates per call.  Atomics to one cache line retire one after the other in L2
+// (about 36 ns each), which would make those few columns the critical path of the whole pass.
+// While a pass runs, the value of a hot column w < kHotWords is therefore represented as
+//     table[w] + sum over s < kShadows of shadow[s][w]
+// with the shadows in a scratch buffer that is zero between calls: a reader sums all copies, a
+// writer adds into the one copy chosen by its workgroup index, so the same-line queue is spread
+// over kShadows lines and no update is delayed or dropped.  A small kernel folds the shadows
+// back into the table (and zeroes them) at the end of the call.
+constexpr int kHotWords = 8;
+constexpr int kShadows = 16;
+
+struct Shadow {
+  float* a;  // [kShadows][kHotWords][d] for table A
+  float* b;  // same for table B
+};
+
+template <int R>
+__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* __restrict__ table,
+                                             const float* __restrict__ shadow, int w, int lane,
+                                             int d) {
+  load_col<R>(x, table + (int64_t)w * d, lane, d);
+  if (w < kHotWords) {
+#pragma unroll 4
+    for (int s = 0; s < kShadows; ++s) {
+      const float* col = shadow + ((int64_t)s * kHotWords + w) * d;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int e = r * kWave + lane;
+        if (r < R - 1 || e < d) x[r] += col[e];
+      }
+    }
   }
+}
+
+// Column that receives the atomics for word w from the workgroup that uses shadow copy `slot`.
+__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int slot,
+                                                 int d) {
+  return w < kHotWords ? shadow + ((int64_t)slot * kHotWords + w) * d : table + (int64_t)w * d;
 }
 
 // Block-level sum of one double per wave, written as one partial per block.

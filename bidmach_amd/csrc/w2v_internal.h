@@ -14,7 +14,20 @@
     default: return hipErrorInvalidValue;                                                  \
   }
 
+#include "w2v_device.h"
+
 namespace w2v {
+
+// Bytes of one shadow buffer (one per table): kShadows copies of kHotWords columns of up to
+// max_rows() floats.  The caller of launch_pos / launch_neg provides both buffers zeroed; the
+// launchers leave them zeroed.
+size_t shadow_bytes();
+
+// Grid size of a persistent kernel: workgroups that fit on the device at once.
+hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t* nwg);
+
+// Adds the shadow copies of the hot columns into A and B and zeroes them.
+hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);
 
 // Number of per-block partial sums an Eval launch over `units` work units writes.
 int64_t eval_partials_needed(int64_t units);
@@ -23,10 +36,11 @@ int64_t eval_partials_needed(int64_t units);
 // `shift` is the caller's maximum window half-width; it sizes the halo a tile stages in LDS.
 // Offsets beyond it are still processed (gathered from memory), so any LB/UB is accepted.
 hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
-                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp);
+                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp,
+                      Shadow shadow);
 
 hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
-                      const int* WB, float* A, float* B, float lrate, float vexp);
+                      const int* WB, float* A, float* B, float lrate, float vexp, Shadow shadow);
 
 // Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
 // and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or

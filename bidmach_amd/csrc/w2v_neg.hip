@@ -8,12 +8,17 @@
 // and every dot product of the group uses the columns as they were when the group started; the
 // nwa + nwb accumulated deltas are scattered once each.
 //
-// One wavefront owns one group.  The nwb B columns and their nwb accumulators stay in registers;
-// A columns stream through CHA at a time (all loads of a chunk issued before its first dot).
-// The CHA*nwb pre-activations of a chunk are parked one per lane so that the sigmoid (a double
-// exp) is evaluated once per chunk; each A delta leaves as float atomics right after its chunk
-// and the B deltas after the last chunk, so every column is read once and updated once per
+// One wavefront owns one group at a time.  The nwb B columns and their nwb accumulators stay in
+// registers; A columns stream through CHA at a time (all loads of a chunk issued before its first
+// dot).  The CHA*nwb pre-activations of a chunk are parked one per lane so that the sigmoid (a
+// double exp) is evaluated once per chunk; each A delta leaves as float atomics right after its
+// chunk and the B deltas after the last chunk, so every column is read once and updated once per
 // group.
+//
+// The update kernel is persistent: a fixed number of workgroups each walk a contiguous range of
+// groups, which bounds the number of groups in flight (and with it the staleness of the Hogwild
+// updates) by the launch size.  The hottest columns are read and updated through their shadow
+// copies (w2v_device.h), so their same-line atomics spread over kShadows lines.
 //
 // The reference reads WA/WB without a validity test (:213-214,220-221); here a negative id
 // skips every pair it takes part in, so a bad id cannot become an out-of-bounds access.
@@ -129,6 +134,101 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
   }
 }
 
+constexpr int kNegWaves = 4;
+constexpr int kNegThreads = kNegWaves * kWave;
+
+template <int R, int MAXB, int CHA>
+__global__ void __launch_bounds__(kNegThreads)
+neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
+                 const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
+                 float lrate, float vexp, int smode, Shadow shadow) {
+  static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slot = blockIdx.x % kShadows;
+
+  const int64_t g_begin = (int64_t)blockIdx.x * groups_per_wg;
+  const int64_t g_end = min(g_begin + groups_per_wg, (int64_t)ngroups);
+
+  for (int64_t unit = g_begin + wave; unit < g_end; unit += kNegWaves) {
+    // Lane k < nwb holds B word k and its scale.
+    int wbl = -1;
+    if (lane < nwb) wbl = WB[unit * nwb + lane];
+    const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
+
+    float b[MAXB][R];
+    float dbb[MAXB][R];
+    int wb[MAXB];
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      wb[k] = -1;
+      if (k < nwb) {
+        wb[k] = read_lane(wbl, k);
+        if (wb[k] >= 0) load_col_hot<R>(b[k], B, shadow.b, wb[k], lane, d);
+        zero_col<R>(dbb[k]);
+      }
+    }
+
+    for (int jbase = 0; jbase < nwa; jbase += kWave) {
+      int wal = -1;
+      if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
+      const float sal = wal >= 0 ? scale_of(wal, vexp, smode) : 0.0f;
+      const int jend = min(nwa - jbase, kWave);
+
+      for (int j0 = 0; j0 < jend; j0 += CHA) {
+        float a[CHA][R];
+        int wa[CHA];
+#pragma unroll
+        for (int c = 0; c < CHA; ++c) {
+          wa[c] = -1;
+          if (j0 + c < jend) {
+            wa[c] = read_lane(wal, j0 + c);
+            if (wa[c] >= 0) load_col_hot<R>(a[c], A, shadow.a, wa[c], lane, d);
+          }
+        }
+        float pre = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CHA; ++c) {
+          if (wa[c] >= 0) {
+#pragma unroll
+            for (int k = 0; k < MAXB; ++k) {
+              if (wb[k] >= 0) {
+                const float s = wave_sum(dot_partial<R>(a[c], b[k]));
+                pre = (lane == c * MAXB + k) ? s : pre;
+              }
+            }
+          }
+        }
+        const float gl = -lrate * sat_sigmoid(pre);
+#pragma unroll
+        for (int c = 0; c < CHA; ++c) {
+          if (wa[c] >= 0) {
+            const float as = read_lane(sal, j0 + c);
+            float daa[R];
+            zero_col<R>(daa);
+#pragma unroll
+            for (int k = 0; k < MAXB; ++k) {
+              if (wb[k] >= 0) {
+                const float g = read_lane(gl, c * MAXB + k);
+                const float bs = read_lane(sbl, k);
+                axpy<R>(dbb[k], bs * g, a[c]);
+                axpy<R>(daa, as * g, b[k]);
+              }
+            }
+            atomic_add_col<R>(scatter_target(A, shadow.a, wa[c], slot, d), daa, lane, d);
+          }
+        }
+      }
+    }
+
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      if (wb[k] >= 0)
+        atomic_add_col<R>(scatter_target(B, shadow.b, wb[k], slot, d), dbb[k], lane, d);
+    }
+  }
+}
+
 constexpr int kMaxNwb = 8;
 int max_nwb() { return kMaxNwb; }
 
@@ -140,40 +240,59 @@ struct NegChunk {
   static constexpr int value = capped < 1 ? 1 : capped;
 };
 
-template <int R, int MAXB, bool TRAIN>
-static hipError_t launch_neg_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
-                                const int* WA, const int* WB, float* A, float* B, float lrate,
-                                float vexp, double floorv, double* partials) {
+template <int R, int MAXB>
+static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
+                                     const int* WA, const int* WB, float* A, float* B,
+                                     double floorv, double* partials) {
   const int64_t per_xcd = blocks_per_xcd(ngroups);
   const dim3 grid((unsigned)(per_xcd * kXcds));
-  hipLaunchKernelGGL((neg_kernel<R, MAXB, NegChunk<R, MAXB>::value, TRAIN>), grid, dim3(kBlock), 0,
-                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, lrate, vexp,
-                     scale_mode(vexp), floorv, partials);
+  hipLaunchKernelGGL((neg_kernel<R, MAXB, NegChunk<R, MAXB>::value, false>), grid, dim3(kBlock), 0,
+                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, 0.0f, 0.0f, kScaleOne,
+                     floorv, partials);
   return hipGetLastError();
+}
+
+template <int R, int MAXB>
+static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
+                                      const int* WA, const int* WB, float* A, float* B,
+                                      float lrate, float vexp, Shadow shadow) {
+  auto kern = neg_train_kernel<R, MAXB, NegChunk<R, MAXB>::value>;
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, &nwg);
+  if (err != hipSuccess) return err;
+  const int64_t max_useful = ((int64_t)ngroups + kNegWaves - 1) / kNegWaves;
+  if (nwg > max_useful) nwg = max_useful;
+  const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
+  nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, nwa, nwb,
+                     groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return launch_fold(stream, A, B, shadow, d);
 }
 
 template <int R, bool TRAIN>
 static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
                                const int* WA, const int* WB, float* A, float* B, float lrate,
-                               float vexp, double floorv, double* partials) {
-  if (nwb <= 2)
-    return launch_neg_rb<R, 2, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, vexp,
-                                      floorv, partials);
-  if (nwb <= 5)
-    return launch_neg_rb<R, 5, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, vexp,
-                                      floorv, partials);
-  if (nwb <= kMaxNwb)
-    return launch_neg_rb<R, kMaxNwb, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate,
-                                            vexp, floorv, partials);
+                               float vexp, double floorv, double* partials, Shadow shadow) {
+#define W2V_NEG_DISPATCH(MAXB_)                                                                  \
+  return TRAIN ? launch_neg_train_rb<R, MAXB_>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, \
+                                               vexp, shadow)                                     \
+               : launch_neg_eval_rb<R, MAXB_>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, floorv, \
+                                              partials)
+  if (nwb <= 2) W2V_NEG_DISPATCH(2);
+  if (nwb <= 5) W2V_NEG_DISPATCH(5);
+  if (nwb <= kMaxNwb) W2V_NEG_DISPATCH(kMaxNwb);
+#undef W2V_NEG_DISPATCH
   return hipErrorInvalidValue;
 }
 
 hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
-                      const int* WB, float* A, float* B, float lrate, float vexp) {
+                      const int* WB, float* A, float* B, float lrate, float vexp, Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R)                                                                                   \
   return launch_neg_r<R, true>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, 0.0,    \
-                               nullptr)
+                               nullptr, shadow)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }
@@ -185,7 +304,7 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
   hipError_t err = hipSuccess;
 #define CALL(R)                                                                                   \
   err = launch_neg_r<R, false>(stream, nrows, ncols, nwa, nwb, WA, WB, const_cast<float*>(A),     \
-                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials);              \
+                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials, Shadow{});    \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL

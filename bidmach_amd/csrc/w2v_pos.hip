@@ -128,9 +128,9 @@ pos_kernel(int d, int ncols, int64_t per_xcd, const int* __restrict__ W,
 
 constexpr int kTileWaves = 8;
 constexpr int kTileThreads = kTileWaves * kWave;
-constexpr int kMaxHalo = 31;  // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
+constexpr int kMaxHalo = 31;       // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
 
-// LDS layout of a tile: a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh]
+// LDS layout of a workgroup: a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh]
 // with dp = R*64 (columns zero-padded so that LDS reads need no bounds test).
 __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
   const size_t dp = (size_t)R * kWave;
@@ -140,9 +140,10 @@ __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
 
 template <int R>
 __global__ void __launch_bounds__(kTileThreads)
-pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t per_xcd, const int* __restrict__ W,
-                const int* __restrict__ LB, const int* __restrict__ UB, float* A, float* B,
-                float lrate, float vexp, int smode) {
+pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg,
+                const int* __restrict__ W, const int* __restrict__ LB,
+                const int* __restrict__ UB, float* A, float* B, float lrate, float vexp,
+                int smode, Shadow shadow) {
   extern __shared__ float lds[];
   constexpr int dp = R * kWave;
   const int lane = threadIdx.x & 63;
@@ -152,132 +153,202 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t per_xcd, const int* __r
   float* const b_t = a_t + (size_t)T * dp;
   float* const G = b_t + (size_t)(T + 2 * Sh) * dp;
   int* const wt = reinterpret_cast<int*>(G + (size_t)T * gw);
+  const int slot = blockIdx.x % kShadows;
 
-  const int64_t tile = xcd_contiguous_block(per_xcd);
-  const int64_t lo64 = tile * T;
-  if (lo64 >= ncols) return;  // whole workgroup leaves together
-  const int lo = (int)lo64;
-  const int hi = min(lo + T, ncols);          // centres [lo, hi)
-  const int hlo = max(lo - Sh, 0);
-  const int hhi = min(hi + Sh, ncols);        // staged positions [hlo, hhi)
-  const int nh = hhi - hlo;
-  const int nc = hi - lo;
+  const int64_t tile_begin = (int64_t)blockIdx.x * tiles_per_wg;
+  const int64_t tile_end = min(tile_begin + tiles_per_wg, ntiles);
 
-  // ---- stage: word ids, B columns of every staged position, A columns of the centres ----
-  for (int c = wave; c < nh; c += kTileWaves) {
-    const int p = hlo + c;
-    const int w = W[p];
-    if (lane == 0) wt[c] = w;
-    if (w >= 0) {
-      float x[R];
-      load_col<R>(x, B + (int64_t)w * d, lane, d);
+  for (int64_t tile = tile_begin; tile < tile_end; ++tile) {
+    const int lo = (int)(tile * T);
+    const int hi = min(lo + T, ncols);          // centres [lo, hi)
+    const int hlo = max(lo - Sh, 0);
+    const int hhi = min(hi + Sh, ncols);        // staged positions [hlo, hhi)
+    const int nh = hhi - hlo;
+    const int nc = hi - lo;
+
+    // ---- stage: word ids, B columns of every staged position, A columns of the centres.
+    //      Two columns per wave are in flight at a time; hot columns include their shadows.
+    for (int c0 = wave; c0 < nh; c0 += 2 * kTileWaves) {
+      const int c1 = c0 + kTileWaves;
+      const int w0 = W[hlo + c0];
+      const int w1 = c1 < nh ? W[hlo + c1] : -1;
+      float x0[R], x1[R];
+      if (w0 >= 0) load_col_hot<R>(x0, B, shadow.b, w0, lane, d);
+      if (w1 >= 0) load_col_hot<R>(x1, B, shadow.b, w1, lane, d);
+      if (lane == 0) {
+        wt[c0] = w0;
+        if (c1 < nh) wt[c1] = w1;
+      }
+      if (w0 >= 0) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) b_t[(size_t)c * dp + r * kWave + lane] = x[r];
-      if (p >= lo && p < hi) {
-        load_col<R>(x, A + (int64_t)w * d, lane, d);
+        for (int r = 0; r < R; ++r) b_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
+      }
+      if (w1 >= 0) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) a_t[(size_t)(p - lo) * dp + r * kWave + lane] = x[r];
+        for (int r = 0; r < R; ++r) b_t[(size_t)c1 * dp + r * kWave + lane] = x1[r];
       }
     }
-  }
-  for (int k = threadIdx.x; k < nc * gw; k += kTileThreads) G[k] = 0.0f;
-  __syncthreads();
+    for (int c0 = wave; c0 < nc; c0 += 2 * kTileWaves) {
+      const int c1 = c0 + kTileWaves;
+      const int w0 = W[lo + c0];
+      const int w1 = c1 < nc ? W[lo + c1] : -1;
+      float x0[R], x1[R];
+      if (w0 >= 0) load_col_hot<R>(x0, A, shadow.a, w0, lane, d);
+      if (w1 >= 0) load_col_hot<R>(x1, A, shadow.a, w1, lane, d);
+      if (w0 >= 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) a_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
+      }
+      if (w1 >= 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) a_t[(size_t)c1 * dp + r * kWave + lane] = x1[r];
+      }
+    }
+    for (int k = threadIdx.x; k < nc * gw; k += kTileThreads) G[k] = 0.0f;
+    __syncthreads();
 
-  // ---- phase 1: one wave per centre ----
-  for (int ci = wave; ci < nc; ci += kTileWaves) {
-    const int i = lo + ci;
-    const int wi = wt[i - hlo];
-    if (wi < 0) continue;
-    const int jlo = max(LB[i], -i);
-    const int jhi = min(UB[i], ncols - 1 - i);
-    float a[R];
+    // ---- phase 1: one wave per centre ----
+    for (int ci = wave; ci < nc; ci += kTileWaves) {
+      const int i = lo + ci;
+      const int wi = wt[i - hlo];
+      if (wi < 0) continue;
+      const int jlo = max(LB[i], -i);
+      const int jhi = min(UB[i], ncols - 1 - i);
+      float a[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) a[r] = a_t[(size_t)ci * dp + r * kWave + lane];
-    float daa[R];
-    zero_col<R>(daa);
-    const float ascale = scale_of(wi, vexp, smode);
-    bool touched = false;
+      for (int r = 0; r < R; ++r) a[r] = a_t[(size_t)ci * dp + r * kWave + lane];
+      float daa[R];
+      zero_col<R>(daa);
+      const float ascale = scale_of(wi, vexp, smode);
+      bool touched = false;
 
-    // Staged part of the window: lane l stands for offset j = l - Sh.
-    {
-      const int j = lane - Sh;
-      const int c = i + j - hlo;  // staged slot of position i + j
-      int wl = -1;
-      if (lane < gw && j != 0 && j >= jlo && j <= jhi) wl = wt[c];
-      const unsigned long long valid = __ballot(wl >= 0);
-      if (valid != 0ull) {
-        float pre = 0.0f;
-        unsigned long long mask = valid;
-        while (mask != 0ull) {
-          const int l = __builtin_ctzll(mask);
-          mask &= mask - 1ull;
-          const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
-          float s = 0.0f;
+      // Staged part of the window: lane l stands for offset j = l - Sh.
+      {
+        const int j = lane - Sh;
+        int wl = -1;
+        if (lane < gw && j != 0 && j >= jlo && j <= jhi) wl = wt[i + j - hlo];
+        const unsigned long long valid = __ballot(wl >= 0);
+        if (valid != 0ull) {
+          float pre = 0.0f;
+          unsigned long long mask = valid;
+          while (mask != 0ull) {
+            const int l = __builtin_ctzll(mask);
+            mask &= mask - 1ull;
+            const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
+            float s = 0.0f;
 #pragma unroll
-          for (int r = 0; r < R; ++r) s = fmaf(a[r], bcol[r * kWave], s);
-          s = wave_sum(s);
-          pre = (lane == l) ? s : pre;
-        }
-        const float gl = lrate * (1.0f - sat_sigmoid(pre));
-        if (wl >= 0) G[ci * gw + lane] = gl;
-        mask = valid;
-        while (mask != 0ull) {
-          const int l = __builtin_ctzll(mask);
-          mask &= mask - 1ull;
-          const float ag = ascale * read_lane(gl, l);
-          const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
+            for (int r = 0; r < R; ++r) s = fmaf(a[r], bcol[r * kWave], s);
+            s = wave_sum(s);
+            pre = (lane == l) ? s : pre;
+          }
+          const float gl = lrate * (1.0f - sat_sigmoid(pre));
+          if (wl >= 0) G[ci * gw + lane] = gl;
+          mask = valid;
+          while (mask != 0ull) {
+            const int l = __builtin_ctzll(mask);
+            mask &= mask - 1ull;
+            const float ag = ascale * read_lane(gl, l);
+            const float* bcol = b_t + (size_t)(i + l - Sh - hlo) * dp + lane;
 #pragma unroll
-          for (int r = 0; r < R; ++r) daa[r] = fmaf(ag, bcol[r * kWave], daa[r]);
+            for (int r = 0; r < R; ++r) daa[r] = fmaf(ag, bcol[r * kWave], daa[r]);
+          }
+          touched = true;
         }
+      }
+
+      // Offsets beyond the staged halo (only when LB/UB exceed the caller's `shift`): one
+      // context at a time, gathered from memory and scattered at once.
+      for (int j = jlo; j <= jhi; ++j) {
+        if (j >= -Sh && j <= Sh) {
+          j = Sh;  // skip the staged range
+          continue;
+        }
+        const int wb = W[i + j];
+        if (wb < 0) continue;
+        float b[R];
+        load_col_hot<R>(b, B, shadow.b, wb, lane, d);
+        const float s = wave_sum(dot_partial<R>(a, b));
+        const float g = lrate * (1.0f - sat_sigmoid(s));
+        axpy<R>(daa, ascale * g, b);
+        atomic_axpy_col<R>(scatter_target(B, shadow.b, wb, slot, d),
+                           scale_of(wb, vexp, smode) * g, a, lane, d);
         touched = true;
       }
+      if (touched) atomic_add_col<R>(scatter_target(A, shadow.a, wi, slot, d), daa, lane, d);
     }
+    __syncthreads();
 
-    // Offsets beyond the staged halo (only when LB/UB exceed the caller's `shift`): one context
-    // at a time, gathered from memory and scattered at once.
-    for (int j = jlo; j <= jhi; ++j) {
-      if (j >= -Sh && j <= Sh) {
-        j = Sh;  // skip the staged range
-        continue;
-      }
-      const int wb = W[i + j];
-      if (wb < 0) continue;
-      float b[R];
-      load_col<R>(b, B + (int64_t)wb * d, lane, d);
-      const float s = wave_sum(dot_partial<R>(a, b));
-      const float g = lrate * (1.0f - sat_sigmoid(s));
-      axpy<R>(daa, ascale * g, b);
-      atomic_axpy_col<R>(B + (int64_t)wb * d, scale_of(wb, vexp, smode) * g, a, lane, d);
-      touched = true;
-    }
-    if (touched) atomic_add_col<R>(A + (int64_t)wi * d, daa, lane, d);
-  }
-  __syncthreads();
-
-  // ---- phase 2: one wave per staged position ----
-  for (int c = wave; c < nh; c += kTileWaves) {
-    const int wp = wt[c];
-    if (wp < 0) continue;
-    const int p = hlo + c;
-    // lane l looks at centre i = p - Sh + l; its g for this position sits at offset p - i
-    const int i = p - Sh + lane;
-    float gl = 0.0f;
-    if (lane < gw && i >= lo && i < hi && i != p) gl = G[(i - lo) * gw + (p - i + Sh)];
-    unsigned long long mask = __ballot(gl != 0.0f);
-    if (mask == 0ull) continue;
-    float dbb[R];
-    zero_col<R>(dbb);
-    while (mask != 0ull) {
-      const int l = __builtin_ctzll(mask);
-      mask &= mask - 1ull;
-      const float g = read_lane(gl, l);
-      const int ci = p - Sh + l - lo;
+    // ---- phase 2: one wave per staged position ----
+    for (int c = wave; c < nh; c += kTileWaves) {
+      const int wp = wt[c];
+      if (wp < 0) continue;
+      const int p = hlo + c;
+      // lane l looks at centre i = p - Sh + l; its g for this position sits at offset p - i
+      const int i = p - Sh + lane;
+      float gl = 0.0f;
+      if (lane < gw && i >= lo && i < hi && i != p) gl = G[(i - lo) * gw + (p - i + Sh)];
+      unsigned long long mask = __ballot(gl != 0.0f);
+      if (mask == 0ull) continue;
+      float dbb[R];
+      zero_col<R>(dbb);
+      while (mask != 0ull) {
+        const int l = __builtin_ctzll(mask);
+        mask &= mask - 1ull;
+        const float g = read_lane(gl, l);
+        const float* acol = a_t + (size_t)(p - Sh + l - lo) * dp + lane;
 #pragma unroll
-      for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, a_t[(size_t)ci * dp + r * kWave + lane], dbb[r]);
+        for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, acol[r * kWave], dbb[r]);
+      }
+      atomic_axpy_col<R>(scatter_target(B, shadow.b, wp, slot, d), scale_of(wp, vexp, smode), dbb,
+                         lane, d);
     }
-    const float bs = scale_of(wp, vexp, smode);
-    atomic_axpy_col<R>(B + (int64_t)wp * d, bs, dbb, lane, d);
+    __syncthreads();
   }
+}
+
+// Adds the shadow copies of hot column w of table t (blockIdx.y) into the table and zeroes them.
+// A column no wave touched has all-zero shadows and is left alone, so the vocabulary may be
+// smaller than kHotWords.
+__global__ void __launch_bounds__(kBlock)
+fold_kernel(float* A, float* B, Shadow shadow, int d) {
+  const int w = blockIdx.x;
+  float* const table = blockIdx.y == 0 ? A : B;
+  float* const sh = blockIdx.y == 0 ? shadow.a : shadow.b;
+  for (int e = threadIdx.x; e < d; e += kBlock) {
+    float sum = 0.0f;
+    bool any = false;
+#pragma unroll
+    for (int s = 0; s < kShadows; ++s) {
+      float* p = sh + ((int64_t)s * kHotWords + w) * d + e;
+      const float v = *p;
+      if (v != 0.0f) {
+        any = true;
+        sum += v;
+        *p = 0.0f;
+      }
+    }
+    if (any) table[(int64_t)w * d + e] += sum;
+  }
+}
+
+size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
+
+hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d) {
+  hipLaunchKernelGGL(fold_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, shadow, d);
+  return hipGetLastError();
+}
+
+hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t* nwg) {
+  int dev = 0, cus = 0, per_cu = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (err != hipSuccess) return err;
+  err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds_bytes);
+  if (err != hipSuccess) return err;
+  if (per_cu < 1) per_cu = 1;
+  *nwg = (int64_t)cus * per_cu;
+  return hipSuccess;
 }
 
 // Folds the per-block partial sums in a fixed order (thread t takes t, t+256, ...; then a
@@ -321,10 +392,11 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
   return hipGetLastError();
 }
 
-// Tile size: the largest power of two (8..64) whose LDS footprint lets three workgroups share a
-// CU; if even 8 tokens need more than one CU's LDS the per-centre kernel is used instead.
+// Tile size: the largest power of two (8..64) whose LDS footprint lets two workgroups share a
+// CU; failing that one workgroup per CU; if even 8 tokens do not fit the per-centre kernel is
+// used instead.
 static int pick_tile(int R, int Sh) {
-  constexpr size_t kShare = 52 * 1024, kLimit = 160 * 1024;
+  constexpr size_t kShare = 80 * 1024, kLimit = 160 * 1024;
   int T = 64;
   while (T > 8 && tile_lds_bytes(R, T, Sh) > kShare) T >>= 1;
   if (tile_lds_bytes(R, T, Sh) > kLimit) return 0;
@@ -334,30 +406,39 @@ static int pick_tile(int R, int Sh) {
 template <int R>
 static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int shift, const int* W,
                                     const int* LB, const int* UB, float* A, float* B, float lrate,
-                                    float vexp) {
+                                    float vexp, Shadow shadow) {
   const int Sh = shift < 0 ? 0 : (shift > kMaxHalo ? kMaxHalo : shift);
   const int T = Sh > 0 ? pick_tile(R, Sh) : 0;
   if (T == 0)
     return launch_pos_r<R, true>(stream, d, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr);
   const size_t lds = tile_lds_bytes(R, T, Sh);
   auto kern = pos_tile_kernel<R>;
+  hipError_t err = hipSuccess;
   if (lds > 48 * 1024) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return err;
   }
+  int64_t nwg = 0;
+  err = persistent_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, &nwg);
+  if (err != hipSuccess) return err;
   const int64_t ntiles = ((int64_t)ncols + T - 1) / T;
-  const int64_t per_xcd = (ntiles + kXcds - 1) / kXcds;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * kXcds)), dim3(kTileThreads), lds, stream, d,
-                     ncols, T, Sh, per_xcd, W, LB, UB, A, B, lrate, vexp, scale_mode(vexp));
-  return hipGetLastError();
+  if (nwg > ntiles) nwg = ntiles;
+  const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
+  nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
+                     ntiles, tiles_per_wg, W, LB, UB, A, B, lrate, vexp, scale_mode(vexp), shadow);
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return launch_fold(stream, A, B, shadow, d);
 }
 
 hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
-                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp) {
+                      const int* LB, const int* UB, float* A, float* B, float lrate, float vexp,
+                      Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R) \
-  return launch_pos_tile_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp)
+  return launch_pos_tile_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, shadow)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }
