@@ -215,6 +215,12 @@ int w2v_set_stream(void* stream) {
 void* w2v_get_stream(void) { return reinterpret_cast<void*>(t_state.stream); }
 int w2v_synchronize(void) { return (int)hipStreamSynchronize(t_state.stream); }
 
+int w2v_set_max_workgroups(int n) {
+  w2v::set_max_workgroups(n);
+  return 0;
+}
+int w2v_get_max_workgroups(void) { return w2v::get_max_workgroups(); }
+
 int w2v_max_rows(void) { return w2v::max_rows(); }
 int w2v_max_nwb(void) { return w2v::max_nwb(); }
 

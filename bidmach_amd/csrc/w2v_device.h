@@ -169,19 +169,19 @@ struct Shadow {
 };
 
 template <int R>
-__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* __restrict__ table,
-                                             const float* __restrict__ shadow, int w, int lane,
-                                             int d) {
+__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
+                                             const float* shadow, int w, int lane, int d) {
   load_col<R>(x, table + (int64_t)w * d, lane, d);
   if (w < kHotWords) {
-#pragma unroll 4
-    for (int s = 0; s < kShadows; ++s) {
-      const float* col = shadow + ((int64_t)s * kHotWords + w) * d;
+    // two shadow copies per trip: enough loads in flight without inflating the register count
+    // of the callers, which inline this many times
+#pragma unroll 1
+    for (int s = 0; s < kShadows; s += 2) {
+      float y0[R], y1[R];
+      load_col<R>(y0, shadow + ((int64_t)s * kHotWords + w) * d, lane, d);
+      load_col<R>(y1, shadow + ((int64_t)(s + 1) * kHotWords + w) * d, lane, d);
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int e = r * kWave + lane;
-        if (r < R - 1 || e < d) x[r] += col[e];
-      }
+      for (int r = 0; r < R; ++r) x[r] += y0[r] + y1[r];
     }
   }
 }

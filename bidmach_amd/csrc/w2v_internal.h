@@ -23,8 +23,14 @@ namespace w2v {
 // launchers leave them zeroed.
 size_t shadow_bytes();
 
-// Grid size of a persistent kernel: workgroups that fit on the device at once.
-hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t* nwg);
+// Grid size of a persistent kernel: the workgroups that fit on the device at once, but no more
+// than `units / min_units_per_wg` (a workgroup walks at least that many work units, so a small
+// minibatch is not spread over the whole device: fewer units in flight means less stale Hogwild
+// updates), and no more than the caller's limit (set_max_workgroups, 0 = none).
+hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
+                           int64_t min_units_per_wg, int64_t* nwg);
+void set_max_workgroups(int n);
+int get_max_workgroups();
 
 // Adds the shadow copies of the hot columns into A and B and zeroes them.
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);

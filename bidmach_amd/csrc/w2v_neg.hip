@@ -136,9 +136,15 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
 
 constexpr int kNegWaves = 4;
 constexpr int kNegThreads = kNegWaves * kWave;
+constexpr int kMinGroupsPerWg = 512;  // a workgroup walks at least this many consecutive groups
+// Waves per SIMD the update kernel is compiled for.  The pass is bound by atomic latency, so it
+// wants waves in flight more than it wants registers per wave.
+#ifndef W2V_NEG_WAVES_PER_EU
+#define W2V_NEG_WAVES_PER_EU 3
+#endif
 
 template <int R, int MAXB, int CHA>
-__global__ void __launch_bounds__(kNegThreads)
+__global__ void __launch_bounds__(kNegThreads, W2V_NEG_WAVES_PER_EU)
 neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
                  const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
                  float lrate, float vexp, int smode, Shadow shadow) {
@@ -232,11 +238,11 @@ neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
 constexpr int kMaxNwb = 8;
 int max_nwb() { return kMaxNwb; }
 
-// A columns gathered per chunk, sized so that b, dbb and the chunk stay near 128 registers.
+// A columns gathered per chunk, sized so that b, dbb and the chunk stay near 100 registers.
 template <int R, int MAXB>
 struct NegChunk {
-  static constexpr int budget = (128 - 2 * MAXB * R) / R;
-  static constexpr int capped = budget > 8 ? 8 : budget;
+  static constexpr int budget = (100 - 2 * MAXB * R) / R;
+  static constexpr int capped = budget > 5 ? 5 : budget;
   static constexpr int value = capped < 1 ? 1 : capped;
 };
 
@@ -258,10 +264,9 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
                                       float lrate, float vexp, Shadow shadow) {
   auto kern = neg_train_kernel<R, MAXB, NegChunk<R, MAXB>::value>;
   int64_t nwg = 0;
-  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, &nwg);
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, ngroups,
+                                   kMinGroupsPerWg, &nwg);
   if (err != hipSuccess) return err;
-  const int64_t max_useful = ((int64_t)ngroups + kNegWaves - 1) / kNegWaves;
-  if (nwg > max_useful) nwg = max_useful;
   const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, nwa, nwb,

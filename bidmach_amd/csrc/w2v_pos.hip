@@ -30,6 +30,8 @@
 // A token therefore costs about (2T + 2Sh)/T columns of atomics instead of 1 + (pairs).
 // All dot products of a tile use the columns as staged (a tile is a small synchronous batch);
 // between tiles the updates are Hogwild, as between the reference's threads.
+#include <atomic>
+
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
@@ -129,6 +131,7 @@ pos_kernel(int d, int ncols, int64_t per_xcd, const int* __restrict__ W,
 constexpr int kTileWaves = 8;
 constexpr int kTileThreads = kTileWaves * kWave;
 constexpr int kMaxHalo = 31;       // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
+constexpr int kMinTilesPerWg = 64; // a workgroup walks at least this many consecutive tiles
 
 // LDS layout of a workgroup: a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh]
 // with dp = R*64 (columns zero-padded so that LDS reads need no bounds test).
@@ -338,7 +341,12 @@ hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, in
   return hipGetLastError();
 }
 
-hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t* nwg) {
+static std::atomic<int> g_max_workgroups{0};
+void set_max_workgroups(int n) { g_max_workgroups.store(n < 0 ? 0 : n); }
+int get_max_workgroups() { return g_max_workgroups.load(); }
+
+hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
+                           int64_t min_units_per_wg, int64_t* nwg) {
   int dev = 0, cus = 0, per_cu = 0;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return err;
@@ -347,7 +355,13 @@ hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, in
   err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds_bytes);
   if (err != hipSuccess) return err;
   if (per_cu < 1) per_cu = 1;
-  *nwg = (int64_t)cus * per_cu;
+  int64_t n = (int64_t)cus * per_cu;
+  const int64_t by_units = (units + min_units_per_wg - 1) / min_units_per_wg;
+  if (n > by_units) n = by_units;
+  const int limit = g_max_workgroups.load();
+  if (limit > 0 && n > limit) n = limit;
+  if (n < 1) n = 1;
+  *nwg = n;
   return hipSuccess;
 }
 
@@ -392,12 +406,13 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
   return hipGetLastError();
 }
 
-// Tile size: the largest power of two (8..64) whose LDS footprint lets two workgroups share a
-// CU; failing that one workgroup per CU; if even 8 tokens do not fit the per-centre kernel is
-// used instead.
+// Tile size: 16 tokens, or 8 if that is what lets two workgroups share a CU's LDS; if even 8
+// tokens do not fit in one CU's LDS the per-centre kernel is used instead.  A tile is a small
+// synchronous batch (all its dot products use the staged columns), so larger tiles would trade
+// fewer atomics for staler updates of the frequent words.
 static int pick_tile(int R, int Sh) {
   constexpr size_t kShare = 80 * 1024, kLimit = 160 * 1024;
-  int T = 64;
+  int T = 16;
   while (T > 8 && tile_lds_bytes(R, T, Sh) > kShare) T >>= 1;
   if (tile_lds_bytes(R, T, Sh) > kLimit) return 0;
   return T;
@@ -419,11 +434,11 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return err;
   }
-  int64_t nwg = 0;
-  err = persistent_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, &nwg);
-  if (err != hipSuccess) return err;
   const int64_t ntiles = ((int64_t)ncols + T - 1) / T;
-  if (nwg > ntiles) nwg = ntiles;
+  int64_t nwg = 0;
+  err = persistent_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, ntiles,
+                        kMinTilesPerWg, &nwg);
+  if (err != hipSuccess) return err;
   const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
   nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,

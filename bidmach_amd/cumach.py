@@ -24,7 +24,8 @@ class W2VLibraryError(RuntimeError):
 
 
 def lib_path():
-    return os.path.join(_HERE, "lib", _LIB_NAME)
+    """Path of the HIP library; BIDMACH_W2V_LIB overrides the in-tree default."""
+    return os.environ.get("BIDMACH_W2V_LIB") or os.path.join(_HERE, "lib", _LIB_NAME)
 
 
 # name -> (restype, argtypes); every symbol include/bidmach_w2v.h declares.
@@ -49,6 +50,8 @@ SYMBOLS = {
     "w2v_set_stream": (_I, [_P]),
     "w2v_get_stream": (_P, []),
     "w2v_synchronize": (_I, []),
+    "w2v_set_max_workgroups": (_I, [_I]),
+    "w2v_get_max_workgroups": (_I, []),
     "w2v_max_rows": (_I, []),
     "w2v_max_nwb": (_I, []),
     "w2v_malloc": (_I, [ctypes.POINTER(_P), _SZ]),
@@ -71,6 +74,14 @@ def load_library(path=None):
     if _lib is not None and path is None:
         return _lib
     p = path or lib_path()
+    # PyTorch-ROCm ships its own copy of the HIP runtime.  If it is going to be used in this
+    # process (it owns the device buffers in the tests and the benchmark) it has to be loaded
+    # first, so that this library binds to the same runtime instance instead of bringing in the
+    # system copy next to it.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     if not os.path.exists(p):
         raise W2VLibraryError(
             "HIP library %s is missing: build it with `python -m bidmach_amd.build` "

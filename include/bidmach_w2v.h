@@ -86,6 +86,14 @@ int w2v_set_stream(void *stream);
 void *w2v_get_stream(void);
 int w2v_synchronize(void);
 
+/* Upper bound on the workgroups of the two update kernels, process-wide (0 = as many as the
+ * device holds, the default).  The update kernels are persistent: each workgroup walks a
+ * contiguous range of the minibatch in order, so this bounds the number of work units in flight
+ * and with it how stale a Hogwild read can be (the reference's CPU path bounds it by its thread
+ * count, BIDMach_CPUMACH.c:21-24). */
+int w2v_set_max_workgroups(int n);
+int w2v_get_max_workgroups(void);
+
 /* Limits of the kernels: largest nrows and largest nwb. */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
