@@ -96,6 +96,9 @@ def main():
     ap.add_argument("--distinct", type=int, default=8,
                     help="number of distinct minibatches generated; steps cycle through them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run one plain 1 GiB device copy before the timed region (gives a "
+                         "kernel of known traffic to scale rocprofv3 FETCH_SIZE/WRITE_SIZE by)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -145,6 +148,13 @@ def main():
                                       A, B, lr / cfg["nneg"], args.vexp), "word2vecNeg")
         if timers:
             timers[1].stop()
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for s in range(Wm):
         step(s)

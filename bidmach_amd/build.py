@@ -16,6 +16,7 @@ OBJ = os.path.join(CSRC, "_obj")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_NAME = "libbidmachhip-linux-x86_64.so"
 LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
+PROBE_PATH = os.path.join(LIB_DIR, "probe_atomics")
 
 SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_api.hip"]
 
@@ -56,7 +57,25 @@ def build(extra_flags=(), verbose=True, out=None):
     subprocess.check_call(cmd)
     if verbose:
         print("built", out)
+    if out == LIB_PATH:
+        build_probe(verbose)
     return out
+
+
+def build_probe(verbose=True):
+    """The stand-alone device probe behind the atomic-scatter ceiling quoted in the design notes."""
+    cmd = [_hipcc(), "-O3", "-std=c++17", "--offload-arch=gfx950", "-munsafe-fp-atomics",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           os.path.join(CSRC, "probe_atomics.hip"), "-o", PROBE_PATH]
+    res = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    if res.returncode != 0:
+        raise subprocess.CalledProcessError(res.returncode, cmd)
+    if verbose:
+        print("built", PROBE_PATH)
+    return PROBE_PATH
 
 
 if __name__ == "__main__":

@@ -1,0 +1,204 @@
+"""Host-side mirror of the minibatch step of BIDMach.networks.Word2Vec around the HIP operators.
+
+What is mirrored (src/main/scala/BIDMach/networks/Word2Vec.scala of the reference):
+  Options         the option names and defaults of Word2Vec.Opts (:574-591) plus the borrowed
+                  dim (models/Model.scala:537), lrate/texp (updaters/Grad.scala:242-243) and
+                  vexp (updaters/ADAGrad.scala:158)
+  init            model matrices: modelmats(0) ~ (U[0,1) - 0.5)/dim, modelmats(1) = 0 (:112-117)
+  wordMats        OOV and subsampling to -1, random window bounds clipped at sentence
+                  boundaries, compaction and permutation of the context words, negatives by the
+                  closed form min(V-1, floor(V * u**(1/(1-wexpt)))) (:214-364)
+  dobatch         learning-rate decay lrate * (pos/firstPos)**(-texp), then procPositives and
+                  procNegatives with A = modelmats(1), B = modelmats(0) (:167-190, :366-402)
+  evalbatch       (epos + eneg/nneg) / #context words (:192-212, :469-523)
+  train           Learner.nextPass' loop: minibatch istep is scored instead of trained on when
+                  (istep - 1) % evalStep == 0, and so is the last one of a pass
+                  (Learner.scala:187-222, evalStep default 11 at :1064)
+
+The arithmetic runs in the HIP library through bidmach_amd.cumach.CUMACH; this module only
+prepares index arrays (numpy, on the host, like the reference's CPU branch `getnegs`) and owns the
+device buffers (torch tensors: plumbing).  Random draws come from numpy, not from BIDMat, so a run
+reproduces the reference's distributions and array contracts, not its random stream.
+"""
+import math
+
+import numpy as np
+
+from . import corpus
+from .cumach import CUMACH, check
+
+
+class Options:
+    """Word2Vec.Opts with the reference's defaults."""
+
+    def __init__(self, **kw):
+        self.nskip = 5
+        self.nneg = 5
+        self.nreuse = 5
+        self.vocabSize = 100000
+        self.wexpt = 0.75
+        self.wsample = 1e-4
+        self.headlen = 10000
+        self.iflip = False
+        self.eqPosNeg = False
+        self.dim = 256
+        self.lrate = 1.0
+        self.texp = 0.5
+        self.vexp = 0.5
+        self.batchSize = 100000
+        self.evalStep = 11
+        self.seed = 0
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("unknown Word2Vec option %r" % k)
+            setattr(self, k, v)
+
+
+class Word2Vec:
+    def __init__(self, opts=None, device="cuda:0"):
+        self.opts = opts or Options()
+        self.device = device
+        self.modelmats = None
+        self.firstPos = -1
+        self.ncols = None
+        self.rng = np.random.Generator(np.random.PCG64(self.opts.seed))
+        self._ret = None
+
+    # ---- Word2Vec.init ------------------------------------------------------------------
+    def init(self, ncols=None, modelmats=None):
+        import torch
+        o = self.opts
+        self.ncols = ncols if ncols is not None else o.batchSize
+        if modelmats is None:
+            m0 = (self.rng.random((o.vocabSize, o.dim), dtype=np.float32) - np.float32(0.5)) \
+                / np.float32(o.dim)
+            m1 = np.zeros((o.vocabSize, o.dim), dtype=np.float32)
+        else:
+            m0, m1 = modelmats
+        # (vocab, dim) C-order == dim x vocab column-major, the layout the operators take
+        self.modelmats = [torch.from_numpy(np.ascontiguousarray(m0)).to(self.device),
+                          torch.from_numpy(np.ascontiguousarray(m1)).to(self.device)]
+        self.expt = 1.0 / (1.0 - o.wexpt)
+        self.salpha = o.wsample * math.log(o.vocabSize)
+        self._ret = torch.zeros(2, dtype=torch.float32, device=self.device)
+        self.firstPos = -1
+
+    # ---- Word2Vec.wordMats (host branch) ------------------------------------------------
+    def wordMats(self, mats):
+        """mats: int32 array 2 x N (row 0 word ids, row 1 sentence ids; swapped if iflip).
+        Returns host arrays (words, lb, ub, trandwords, contextwords)."""
+        o = self.opts
+        wordsens = np.asarray(mats)
+        words = (wordsens[1] if o.iflip else wordsens[0]).astype(np.int32)
+        sentence = wordsens[0] if o.iflip else wordsens[1]
+        n = words.shape[0]
+        wgood = words < o.vocabSize
+        wrat = (words.astype(np.float32) + np.float32(1.0)) * np.float32(self.salpha)
+        wrat = np.sqrt(wrat) + wrat
+        wgood &= self.rng.random(n, dtype=np.float32) < wrat
+        words = np.where(wgood, words, -1).astype(np.int32)
+
+        ubrand = np.minimum(o.nskip, (self.rng.random(n, dtype=np.float32) * o.nskip)
+                            .astype(np.int32) + 1).astype(np.int32)
+        lbrand = -ubrand
+        # nearest sentence boundaries: position inside the run of equal sentence ids
+        idx = np.arange(n, dtype=np.int64)
+        change = np.flatnonzero(sentence[1:] != sentence[:-1]) + 1
+        starts = np.concatenate(([0], change))
+        ends = np.concatenate((change, [n])) - 1
+        seg = np.searchsorted(starts, idx, side="right") - 1
+        lb = np.maximum(lbrand, (starts[seg] - idx)).astype(np.int32)
+        ub = np.minimum(ubrand, (ends[seg] - idx)).astype(np.int32)
+
+        ctx = corpus.valid_context_words(words, lb, ub)
+        ngroups = ctx.shape[0] // o.nreuse
+        ctx = self.rng.permutation(ctx)[: ngroups * o.nreuse].astype(np.int32)
+        u = self.rng.random(ngroups * o.nneg, dtype=np.float32)
+        negs = np.minimum(o.vocabSize - 1,
+                          (o.vocabSize * np.power(u, np.float32(self.expt))).astype(np.int64))
+        return words, lb, ub, negs.astype(np.int32), ctx
+
+    def _dev(self, x):
+        import torch
+        return torch.from_numpy(np.ascontiguousarray(x)).to(self.device)
+
+    # ---- the four dispatchers (Word2Vec.scala:366-402, 469-523) --------------------------
+    def procPositives(self, nskip, words, lb, ub, model1, model2, lrate, vexp):
+        nrows = model1.shape[1]
+        check(CUMACH.word2vecPos(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
+                                 lrate, vexp), "word2vecPos")
+
+    def procNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb, lrate, vexp):
+        nrows = modela.shape[1]
+        check(CUMACH.word2vecNeg(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb, modela,
+                                 modelb, lrate, vexp), "word2vecNeg")
+
+    def evalPositives(self, nskip, words, lb, ub, model1, model2):
+        nrows = model1.shape[1]
+        self._ret[0:1].zero_()                                  # retEvalPos.clear (:476)
+        check(CUMACH.word2vecEvalPos(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
+                                     self._ret[0:1]), "word2vecEvalPos")
+        return float(self._ret[0].item())
+
+    def evalNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb):
+        nrows = modela.shape[1]
+        self._ret[1:2].zero_()
+        check(CUMACH.word2vecEvalNeg(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
+                                     modela, modelb, self._ret[1:2]), "word2vecEvalNeg")
+        return float(self._ret[1].item())
+
+    # ---- Word2Vec.dobatch / evalbatch ---------------------------------------------------
+    def dobatch(self, mats, ipass, pos):
+        o = self.opts
+        if np.asarray(mats).shape[1] != self.ncols:
+            return                                              # odd-sized minibatch: skipped (:169)
+        if self.firstPos < 0:
+            self.firstPos = pos
+        nsteps = float(pos) / float(self.firstPos)
+        lrate = float(o.lrate) * math.pow(nsteps, -o.texp)
+        words, lb, ub, trandwords, goodwords = self.wordMats(mats)
+        lrpos = lrate
+        lrneg = lrpos if o.eqPosNeg else lrpos / o.nneg
+        dw, dlb, dub = self._dev(words), self._dev(lb), self._dev(ub)
+        self.procPositives(o.nskip, dw, dlb, dub, self.modelmats[1], self.modelmats[0], lrpos,
+                           o.vexp)
+        if goodwords.shape[0] > 0:
+            self.procNegatives(o.nneg, o.nreuse, self._dev(trandwords), self._dev(goodwords),
+                               self.modelmats[1], self.modelmats[0], lrneg, o.vexp)
+
+    def evalbatch(self, mats, ipass, pos):
+        o = self.opts
+        if np.asarray(mats).shape[1] != self.ncols:
+            return 0.0                                          # row(0) (:211)
+        words, lb, ub, trandwords, goodwords = self.wordMats(mats)
+        if goodwords.shape[0] == 0:
+            return 0.0
+        epos = self.evalPositives(o.nskip, self._dev(words), self._dev(lb), self._dev(ub),
+                                  self.modelmats[1], self.modelmats[0])
+        eneg = self.evalNegatives(o.nneg, o.nreuse, self._dev(trandwords), self._dev(goodwords),
+                                  self.modelmats[1], self.modelmats[0])
+        return (epos + eneg / (1 if o.eqPosNeg else o.nneg)) / goodwords.shape[0]
+
+    # ---- Learner.nextPass, reduced to what Word2Vec uses (no updater, no mixins) ---------
+    def train(self, stream, npasses=1):
+        """stream: int32 array 2 x total.  Returns [(position, held-out score)], one entry per
+        evalStep-th minibatch, as Learner collects in `results` (Learner.scala:276)."""
+        o = self.opts
+        stream = np.asarray(stream)
+        if self.modelmats is None:
+            self.init(o.batchSize)
+        results = []
+        here = 0
+        for ipass in range(npasses):
+            istep = 0
+            starts = list(range(0, stream.shape[1] - o.batchSize + 1, o.batchSize))
+            for s in starts:
+                mats = stream[:, s:s + o.batchSize]
+                here += o.batchSize
+                last = s == starts[-1]
+                if (istep >= 1 and (istep - 1) % o.evalStep == 0) or (istep > 0 and last):
+                    results.append((here, self.evalbatch(mats, ipass, here)))
+                else:
+                    self.dobatch(mats, ipass, here)
+                istep += 1
+        return results
