@@ -22,6 +22,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE on this same command (summaries under profiles/), scaled by what the same
+# counters read for a plain copy of known size in the same run (FETCH x2.0, WRITE x1.0).
+MEASURED_TRAFFIC_BYTES = {
+    "sgns_v1m_d300_w5_neg5_fp32": {"neg_kernel": 36.09e9, "pos_kernel": 6.61e9},
+}
+
 WORKLOADS = {
     # name: vocab, dim, tokens per minibatch, window half-width, nneg, nreuse, zipf exponent
     "sgns_v1m_d300_w5_neg5_fp32": dict(vocab=1_000_000, dim=300, tokens=1_000_000, skip=5, nneg=5,
@@ -205,7 +212,8 @@ def main():
         # the negative pass moves ~63% of the step's algorithmic bytes: it is the dominant kernel
         "roofline": {"bound": "hbm", "kernel": "neg_kernel", "achieved": neg_gbps,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": neg_gbps / HBM_PEAK_GBPS,
-                     "traffic": None, "algorithmic_bytes_per_launch": avg_neg_b,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get("neg_kernel"),
+                     "algorithmic_bytes_per_launch": avg_neg_b,
                      "avg_launch_ms": avg_neg_ms},
         "kernels": {
             "pos_kernel": {"avg_launch_ms": avg_pos_ms, "algorithmic_bytes_per_launch": avg_pos_b,

@@ -33,9 +33,10 @@ extern "C" {
 /* Replaces word2vecPos, MatKernel.hpp:77 / DNN127.cu:1389-1420; arithmetic of
  * BIDMach_CPUMACH.c:10-78.  ncols tokens; token i with W[i] >= 0 is a centre word whose window
  * is the offsets j in [LB[i], UB[i]], j != 0, 0 <= i+j < ncols, W[i+j] >= 0.  A is indexed by the
- * centre word, B by the context word; both are updated in place.  `shift` (the reference's
- * template selector, the maximum window half-width) is accepted and not needed: any window
- * width works. */
+ * centre word, B by the context word; both are updated in place.  `shift` is the caller's maximum
+ * window half-width (the reference's template selector, Word2Vec.scala:373 passes nskip); here
+ * it only sizes the halo a tile of tokens stages on chip, so any value gives the same result and
+ * any window width works. */
 int word2vecPos(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A, float *B,
                 float lrate, float vexp);
 
