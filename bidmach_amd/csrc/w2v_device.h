@@ -158,10 +158,16 @@ __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float a
 //     table[w] + sum over s < kShadows of shadow[s][w]
 // with the shadows in a scratch buffer that is zero between calls: a reader sums all copies, a
 // writer adds into the one copy chosen by its workgroup index, so the same-line queue is spread
-// over kShadows lines and no update is delayed or dropped.  A small kernel folds the shadows
-// back into the table (and zeroes them) at the end of the call.
+// over several lines and no update is delayed or dropped.  A small kernel folds the shadows
+// back into the table (and zeroes them) at the end of the call.  The number of copies follows
+// the Zipf law: 16 for word 0, 8 for words 1-2, 4 for words 3-6, 2 for word 7, so every hot
+// line sees about the same queue and readers do not sum more copies than needed.
 constexpr int kHotWords = 8;
 constexpr int kShadows = 16;
+
+__device__ __forceinline__ int shadow_copies(int w) {
+  return kShadows >> (31 - __builtin_clz(w + 1));
+}
 
 struct Shadow {
   float* a;  // [kShadows][kHotWords][d] for table A
@@ -175,8 +181,9 @@ __device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
   if (w < kHotWords) {
     // two shadow copies per trip: enough loads in flight without inflating the register count
     // of the callers, which inline this many times
+    const int copies = shadow_copies(w);
 #pragma unroll 1
-    for (int s = 0; s < kShadows; s += 2) {
+    for (int s = 0; s < copies; s += 2) {
       float y0[R], y1[R];
       load_col<R>(y0, shadow + ((int64_t)s * kHotWords + w) * d, lane, d);
       load_col<R>(y1, shadow + ((int64_t)(s + 1) * kHotWords + w) * d, lane, d);
@@ -186,10 +193,12 @@ __device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
   }
 }
 
-// Column that receives the atomics for word w from the workgroup that uses shadow copy `slot`.
-__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int slot,
+// Column that receives the atomics for word w from workgroup number `wg`.
+__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int wg,
                                                  int d) {
-  return w < kHotWords ? shadow + ((int64_t)slot * kHotWords + w) * d : table + (int64_t)w * d;
+  if (w >= kHotWords) return table + (int64_t)w * d;
+  const int slot = wg & (shadow_copies(w) - 1);
+  return shadow + ((int64_t)slot * kHotWords + w) * d;
 }
 
 // Block-level sum of one double per wave, written as one partial per block.

@@ -27,11 +27,12 @@
 
 namespace w2v {
 
-template <int R, int MAXB, int CHA, bool TRAIN>
+// Forward-only twin: sum over the group's pairs of log(max(1 - sigmoid(s), floor)).
+template <int R, int MAXB, int CHA>
 __global__ void __launch_bounds__(kBlock)
-neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __restrict__ WA,
-           const int* __restrict__ WB, float* A, float* B, float lrate, float vexp, int smode,
-           double floorv, double* __restrict__ partials) {
+neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __restrict__ WA,
+                const int* __restrict__ WB, const float* __restrict__ A,
+                const float* __restrict__ B, double floorv, double* __restrict__ partials) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -39,13 +40,9 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
   double lsum = 0.0;
 
   if (unit < ngroups) {
-    // Lane k < nwb holds B word k and its scale.
     int wbl = -1;
     if (lane < nwb) wbl = WB[unit * nwb + lane];
-    const float sbl = (TRAIN && wbl >= 0) ? scale_of(wbl, vexp, smode) : 0.0f;
-
     float b[MAXB][R];
-    float dbb[MAXB][R];
     int wb[MAXB];
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
@@ -53,17 +50,12 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
       if (k < nwb) {
         wb[k] = read_lane(wbl, k);
         if (wb[k] >= 0) load_col<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
-        if (TRAIN) zero_col<R>(dbb[k]);
       }
     }
-
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
-      // Lane l holds A word jbase+l and its scale.
       int wal = -1;
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
-      const float sal = (TRAIN && wal >= 0) ? scale_of(wal, vexp, smode) : 0.0f;
       const int jend = min(nwa - jbase, kWave);
-
       for (int j0 = 0; j0 < jend; j0 += CHA) {
         float a[CHA][R];
         int wa[CHA];
@@ -75,8 +67,7 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
             if (wa[c] >= 0) load_col<R>(a[c], A + (int64_t)wa[c] * d, lane, d);
           }
         }
-        // Pre-activation of (c, k) parks in lane c*MAXB + k; lanes without a valid pair keep a
-        // marker below the lower clamp and are masked out afterwards.
+        // Pre-activation of (c, k) parks in lane c*MAXB + k; only those lanes contribute.
         float pre = 0.0f;
         bool live = false;
 #pragma unroll
@@ -93,45 +84,11 @@ neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __r
             }
           }
         }
-        const float sg = sat_sigmoid(pre);
-        if (TRAIN) {
-          const float gl = -lrate * sg;
-#pragma unroll
-          for (int c = 0; c < CHA; ++c) {
-            if (wa[c] >= 0) {
-              const float as = read_lane(sal, j0 + c);
-              float daa[R];
-              zero_col<R>(daa);
-#pragma unroll
-              for (int k = 0; k < MAXB; ++k) {
-                if (wb[k] >= 0) {
-                  const float g = read_lane(gl, c * MAXB + k);
-                  const float bs = read_lane(sbl, k);
-                  axpy<R>(dbb[k], bs * g, a[c]);
-                  axpy<R>(daa, as * g, b[k]);
-                }
-              }
-              atomic_add_col<R>(A + (int64_t)wa[c] * d, daa, lane, d);
-            }
-          }
-        } else {
-          if (live) lsum += log(fmax(1.0 - (double)sg, floorv));
-        }
-      }
-    }
-
-    if (TRAIN) {
-#pragma unroll
-      for (int k = 0; k < MAXB; ++k) {
-        if (wb[k] >= 0) atomic_add_col<R>(B + (int64_t)wb[k] * d, dbb[k], lane, d);
+        if (live) lsum += log(fmax(1.0 - (double)sat_sigmoid(pre), floorv));
       }
     }
   }
-
-  if (!TRAIN) {
-    const double wsum = wave_sum_f64(lsum);
-    block_store_partial(wsum, partials);
-  }
+  block_store_partial(wave_sum_f64(lsum), partials);
 }
 
 constexpr int kNegWaves = 4;
@@ -151,7 +108,7 @@ neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int slot = blockIdx.x % kShadows;
+  const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
   const int64_t g_begin = (int64_t)blockIdx.x * groups_per_wg;
   const int64_t g_end = min(g_begin + groups_per_wg, (int64_t)ngroups);
@@ -252,9 +209,8 @@ static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int
                                      double floorv, double* partials) {
   const int64_t per_xcd = blocks_per_xcd(ngroups);
   const dim3 grid((unsigned)(per_xcd * kXcds));
-  hipLaunchKernelGGL((neg_kernel<R, MAXB, NegChunk<R, MAXB>::value, false>), grid, dim3(kBlock), 0,
-                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, 0.0f, 0.0f, kScaleOne,
-                     floorv, partials);
+  hipLaunchKernelGGL((neg_eval_kernel<R, MAXB, NegChunk<R, MAXB>::value>), grid, dim3(kBlock), 0,
+                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, floorv, partials);
   return hipGetLastError();
 }
 

@@ -156,7 +156,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
   float* const b_t = a_t + (size_t)T * dp;
   float* const G = b_t + (size_t)(T + 2 * Sh) * dp;
   int* const wt = reinterpret_cast<int*>(G + (size_t)T * gw);
-  const int slot = blockIdx.x % kShadows;
+  const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
   const int64_t tile_begin = (int64_t)blockIdx.x * tiles_per_wg;
   const int64_t tile_end = min(tile_begin + tiles_per_wg, ntiles);

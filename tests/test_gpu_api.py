@@ -1,0 +1,165 @@
+"""The C ABI used the way a host without a HIP binding of its own would use it: device buffers
+through w2v_malloc / w2v_memcpy_*, timers, streams, and concurrent host threads (needs an MI355X)."""
+import ctypes
+import threading
+
+import numpy as np
+import pytest
+
+from bidmach_amd import corpus
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import torch
+    assert torch.cuda.is_available()
+    from bidmach_amd.cumach import load_library
+    return load_library()
+
+
+class DevBuf:
+    """A device buffer owned through the library."""
+
+    def __init__(self, lib, host):
+        self.lib = lib
+        self.host = np.ascontiguousarray(host)
+        self.ptr = ctypes.c_void_p()
+        assert lib.w2v_malloc(ctypes.byref(self.ptr), self.host.nbytes) == 0
+        assert lib.w2v_memcpy_h2d(self.ptr, self.host.ctypes.data, self.host.nbytes) == 0
+
+    def download(self):
+        out = np.empty_like(self.host)
+        assert self.lib.w2v_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes) == 0
+        return out
+
+    def free(self):
+        assert self.lib.w2v_free(self.ptr) == 0
+
+
+def test_whole_step_through_library_owned_buffers(lib, oracle):
+    rng = np.random.default_rng(5)
+    d, V, skip, nwa, nwb = 300, 9000, 5, 5, 5
+    A = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    W, LB, UB = corpus.collision_free_pos(150, skip, V, rng)
+    WA, WB = corpus.collision_free_neg(150, nwa, nwb, V, rng)
+    bufs = {k: DevBuf(lib, v) for k, v in dict(A=A, B=B, W=W, LB=LB, UB=UB, WA=WA, WB=WB).items()}
+    ret = DevBuf(lib, np.zeros(2, np.float32))
+    p = {k: b.ptr for k, b in bufs.items()}
+    n = W.shape[0]
+    assert lib.word2vecPos(d, n, skip, p["W"], p["LB"], p["UB"], p["A"], p["B"], 0.025, 0.5) == 0
+    assert lib.word2vecNeg(d, 150, nwa, nwb, p["WA"], p["WB"], p["A"], p["B"], 0.005, 0.5) == 0
+    assert lib.w2v_memset(ret.ptr, 0, 8) == 0
+    assert lib.word2vecEvalPos(d, n, skip, p["W"], p["LB"], p["UB"], p["A"], p["B"], ret.ptr) == 0
+    assert lib.word2vecEvalNeg(d, 150, nwa, nwb, p["WA"], p["WB"], p["A"], p["B"],
+                               ret.ptr.value + 4) == 0
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecPos(d, n, skip, W, LB, UB, Ao, Bo, 0.025, 0.5, 1)
+    oracle.word2vecNeg(d, 150, nwa, nwb, WA, WB, Ao, Bo, 0.005, 0.5, 1)
+    assert np.abs(bufs["A"].download() - Ao).max() <= 1e-4
+    assert np.abs(bufs["B"].download() - Bo).max() <= 1e-4
+    r = ret.download()
+    assert r[0] == pytest.approx(oracle.word2vecEvalPos(d, n, skip, W, LB, UB, Ao, Bo, 1), rel=1e-5)
+    assert r[1] == pytest.approx(oracle.word2vecEvalNeg(d, 150, nwa, nwb, WA, WB, Ao, Bo, 1),
+                                 rel=1e-5)
+    for b in list(bufs.values()) + [ret]:
+        b.free()
+
+
+def test_async_calls_timers_and_stream(lib, oracle):
+    import torch
+    from bidmach_amd.cumach import CUMACH, Timer, synchronize
+    rng = np.random.default_rng(6)
+    d, V, G = 128, 4000, 300
+    A = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    WA, WB = corpus.collision_free_neg(G, 5, 5, V, rng)
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    WAd, WBd = torch.from_numpy(WA).cuda(), torch.from_numpy(WB).cuda()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()                       # default priority
+    assert lib.w2v_get_stream() is None
+    try:
+        assert lib.w2v_set_stream(stream.cuda_stream) == 0
+        assert lib.w2v_get_stream() == stream.cuda_stream
+        t = Timer()
+        t.start()
+        assert CUMACH.word2vecNegAsync(d, G, 5, 5, WAd, WBd, Ad, Bd, 0.01, 0.0) == 0
+        t.stop()
+        ms = t.elapsed_ms()
+        synchronize()
+        assert 0.0 < ms < 1000.0
+    finally:
+        lib.w2v_set_stream(None)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, 5, 5, WA, WB, Ao, Bo, 0.01, 0.0, 1)
+    assert np.abs(Ad.cpu().numpy() - Ao).max() <= 1e-4
+    assert np.abs(Bd.cpu().numpy() - Bo).max() <= 1e-4
+
+
+def test_two_host_threads_call_concurrently(lib, oracle):
+    """Each host thread has its own stream state and scratch; results are independent."""
+    import torch
+    from bidmach_amd.cumach import CUMACH
+    rng = np.random.default_rng(7)
+    d, V, skip = 100, 6000, 5
+    jobs = []
+    for t in range(2):
+        A = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+        B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+        W, LB, UB = corpus.collision_free_pos(250, skip, V, rng)
+        jobs.append(dict(A=A, B=B, W=W, LB=LB, UB=UB,
+                         dev={k: torch.from_numpy(v).cuda()
+                              for k, v in dict(A=A, B=B, W=W, LB=LB, UB=UB).items()},
+                         ret=torch.zeros(1, dtype=torch.float64, device="cuda"), err=[]))
+    torch.cuda.synchronize()
+
+    def work(j):
+        dv = j["dev"]
+        for _ in range(5):
+            j["err"].append(CUMACH.word2vecPos(d, j["W"].shape[0], skip, dv["W"], dv["LB"],
+                                               dv["UB"], dv["A"], dv["B"], 0.01, 0.5))
+        j["err"].append(CUMACH.word2vecEvalPosF64(d, j["W"].shape[0], skip, dv["W"], dv["LB"],
+                                                  dv["UB"], dv["A"], dv["B"], j["ret"]))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for j in jobs:
+        assert j["err"] == [0] * 6
+        Ao, Bo = j["A"].copy(), j["B"].copy()
+        for _ in range(5):
+            oracle.word2vecPos(d, j["W"].shape[0], skip, j["W"], j["LB"], j["UB"], Ao, Bo, 0.01,
+                               0.5, 1)
+        assert np.abs(j["dev"]["A"].cpu().numpy() - Ao).max() <= 1e-4
+        assert np.abs(j["dev"]["B"].cpu().numpy() - Bo).max() <= 1e-4
+        want = oracle.word2vecEvalPos(d, j["W"].shape[0], skip, j["W"], j["LB"], j["UB"], Ao, Bo, 1)
+        assert float(j["ret"].item()) == pytest.approx(want, rel=1e-5)
+
+
+def test_max_workgroups_knob_does_not_change_results(lib, oracle):
+    import torch
+    from bidmach_amd.cumach import CUMACH
+    rng = np.random.default_rng(8)
+    d, V, G = 300, 30000, 2000
+    A = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    WA, WB = corpus.collision_free_neg(G, 5, 5, V, rng)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, 5, 5, WA, WB, Ao, Bo, 0.01, 0.5, 1)
+    assert lib.w2v_get_max_workgroups() == 0
+    try:
+        for limit in (1, 7, 0):
+            lib.w2v_set_max_workgroups(limit)
+            assert lib.w2v_get_max_workgroups() == limit
+            Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+            assert CUMACH.word2vecNeg(d, G, 5, 5, torch.from_numpy(WA).cuda(),
+                                      torch.from_numpy(WB).cuda(), Ad, Bd, 0.01, 0.5) == 0
+            assert np.abs(Ad.cpu().numpy() - Ao).max() <= 1e-4
+            assert np.abs(Bd.cpu().numpy() - Bo).max() <= 1e-4
+    finally:
+        lib.w2v_set_max_workgroups(0)
