@@ -10,6 +10,7 @@
 namespace {
 
 constexpr int kMaxDevices = 64;
+constexpr int kNoIdLimit = 0x7FFFFFFF;
 
 struct ThreadState {
   hipStream_t stream = nullptr;
@@ -102,17 +103,17 @@ int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A
                 sync);
 }
 
-int neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
-             float lrate, float vexp, bool sync) {
-  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb())
+int neg_impl(int nrows, int ncols, int idlimit, int nwa, int nwb, int* WA, int* WB, float* A,
+             float* B, float lrate, float vexp, bool sync) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || idlimit < 0)
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp,
-                                shadow),
+  return finish(w2v::launch_neg(t_state.stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B,
+                                lrate, vexp, shadow),
                 sync);
 }
 
@@ -159,7 +160,12 @@ int word2vecPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float
 
 int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
                 float lrate, float vexp) {
-  return neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, true);
+  return neg_impl(nrows, ncols, kNoIdLimit, nwa, nwb, WA, WB, A, B, lrate, vexp, true);
+}
+
+int word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, int* WA, int* WB, float* A,
+                    float* B, float lrate, float vexp) {
+  return neg_impl(nrows, ncols, nwords, nwa, nwb, WA, WB, A, B, lrate, vexp, true);
 }
 
 int word2vecEvalPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
@@ -191,7 +197,7 @@ int word2vecPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* UB, 
 
 int word2vecNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
                      float lrate, float vexp) {
-  return neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, false);
+  return neg_impl(nrows, ncols, kNoIdLimit, nwa, nwb, WA, WB, A, B, lrate, vexp, false);
 }
 
 int word2vecEvalPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A,

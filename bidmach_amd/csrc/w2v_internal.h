@@ -45,8 +45,10 @@ hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const
                       const int* LB, const int* UB, float* A, float* B, float lrate, float vexp,
                       Shadow shadow);
 
-hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
-                      const int* WB, float* A, float* B, float lrate, float vexp, Shadow shadow);
+// Word ids >= idlimit (and negative ids) are skipped with every pair they take part in.
+hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                      const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
+                      Shadow shadow);
 
 // Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
 // and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or

@@ -102,7 +102,7 @@ constexpr int kMinGroupsPerWg = 512;  // a workgroup walks at least this many co
 
 template <int R, int MAXB, int CHA>
 __global__ void __launch_bounds__(kNegThreads, W2V_NEG_WAVES_PER_EU)
-neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
+neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t groups_per_wg,
                  const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
                  float lrate, float vexp, int smode, Shadow shadow) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
@@ -117,6 +117,7 @@ neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
     // Lane k < nwb holds B word k and its scale.
     int wbl = -1;
     if (lane < nwb) wbl = WB[unit * nwb + lane];
+    if (wbl >= idlimit) wbl = -1;  // word2vecNegFilt: ids beyond the resident columns are skipped
     const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
 
     float b[MAXB][R];
@@ -135,6 +136,7 @@ neg_train_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
       int wal = -1;
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
+      if (wal >= idlimit) wal = -1;
       const float sal = wal >= 0 ? scale_of(wal, vexp, smode) : 0.0f;
       const int jend = min(nwa - jbase, kWave);
 
@@ -215,8 +217,8 @@ static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int
 }
 
 template <int R, int MAXB>
-static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
-                                      const int* WA, const int* WB, float* A, float* B,
+static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, int idlimit, int nwa,
+                                      int nwb, const int* WA, const int* WB, float* A, float* B,
                                       float lrate, float vexp, Shadow shadow) {
   auto kern = neg_train_kernel<R, MAXB, NegChunk<R, MAXB>::value>;
   int64_t nwg = 0;
@@ -225,20 +227,20 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   if (err != hipSuccess) return err;
   const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
-  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, nwa, nwb,
-                     groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, idlimit,
+                     nwa, nwb, groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
   return launch_fold(stream, A, B, shadow, d);
 }
 
 template <int R, bool TRAIN>
-static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
+static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
                                const int* WA, const int* WB, float* A, float* B, float lrate,
                                float vexp, double floorv, double* partials, Shadow shadow) {
 #define W2V_NEG_DISPATCH(MAXB_)                                                                  \
-  return TRAIN ? launch_neg_train_rb<R, MAXB_>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, lrate, \
-                                               vexp, shadow)                                     \
+  return TRAIN ? launch_neg_train_rb<R, MAXB_>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, A, \
+                                               B, lrate, vexp, shadow)                           \
                : launch_neg_eval_rb<R, MAXB_>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, floorv, \
                                               partials)
   if (nwb <= 2) W2V_NEG_DISPATCH(2);
@@ -248,12 +250,13 @@ static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int nwa, 
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb, const int* WA,
-                      const int* WB, float* A, float* B, float lrate, float vexp, Shadow shadow) {
+hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                      const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
+                      Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R)                                                                                   \
-  return launch_neg_r<R, true>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, 0.0,    \
-                               nullptr, shadow)
+  return launch_neg_r<R, true>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp, \
+                               0.0, nullptr, shadow)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }
@@ -264,7 +267,7 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
   const int rounds = (nrows + kWave - 1) / kWave;
   hipError_t err = hipSuccess;
 #define CALL(R)                                                                                   \
-  err = launch_neg_r<R, false>(stream, nrows, ncols, nwa, nwb, WA, WB, const_cast<float*>(A),     \
+  err = launch_neg_r<R, false>(stream, nrows, ncols, 0, nwa, nwb, WA, WB, const_cast<float*>(A),  \
                                const_cast<float*>(B), 0.0f, 0.0f, floorv, partials, Shadow{});    \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)

@@ -37,6 +37,7 @@ _ENEG = [_I, _I, _I, _I, _P, _P, _P, _P, _P]
 SYMBOLS = {
     "word2vecPos": (_I, _POS),
     "word2vecNeg": (_I, _NEG),
+    "word2vecNegFilt": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P, _F, _F]),
     "word2vecEvalPos": (_I, _EPOS),
     "word2vecEvalNeg": (_I, _ENEG),
     "word2vecEvalPosF64": (_I, _EPOS),
@@ -139,6 +140,12 @@ class CUMACH:
     def word2vecNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp):
         return load_library().word2vecNeg(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB), _ptr(A),
                                           _ptr(B), lrate, vexp)
+
+    @staticmethod
+    def word2vecNegFilt(nrows, ncols, nwords, nwa, nwb, WA, WB, A, B, lrate, vexp):
+        """CUMACH.java:94."""
+        return load_library().word2vecNegFilt(nrows, ncols, nwords, nwa, nwb, _ptr(WA), _ptr(WB),
+                                              _ptr(A), _ptr(B), lrate, vexp)
 
     @staticmethod
     def word2vecEvalPos(nrows, ncols, shift, W, LB, UB, A, B, retVal):

@@ -46,6 +46,13 @@ int word2vecPos(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float
 int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A, float *B,
                 float lrate, float vexp);
 
+/* Replaces word2vecNegFilt, MatKernel.hpp:81 / DNN127.cu:670-823,1454-1483 (CUMACH.java:94; used by
+ * the reference when only the first `nwords` columns of a larger model are resident on the GPU,
+ * Word2Vec.scala:448).  As word2vecNeg, but a word id >= nwords is skipped together with every
+ * pair it takes part in (DNN127.cu:690-711); A and B hold nwords columns. */
+int word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, int *WA, int *WB, float *A,
+                    float *B, float lrate, float vexp);
+
 /* Replaces word2vecEvalPos, MatKernel.hpp:83 / DNN127.cu:1485-1516; arithmetic of
  * BIDMach_CPUMACH.c:368-427.  Adds sum(log(max(sigmoid(a.b), floor))) over the valid pairs into
  * the device float Retval[0] (the caller clears it first, Word2Vec.scala:476). */

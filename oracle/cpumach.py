@@ -41,6 +41,8 @@ def _load():
     lib.oracle_word2vecPos.restype = None
     lib.oracle_word2vecNeg.argtypes = [ci, ci, ci, ci, ip, ip, fp, fp, cf, cf, ci]
     lib.oracle_word2vecNeg.restype = None
+    lib.oracle_word2vecNegFilt.argtypes = [ci, ci, ci, ci, ci, ip, ip, fp, fp, cf, cf, ci]
+    lib.oracle_word2vecNegFilt.restype = None
     lib.oracle_word2vecEvalPos.argtypes = [ci, ci, ci, ip, ip, ip, fp, fp, cd, ci]
     lib.oracle_word2vecEvalPos.restype = cd
     lib.oracle_word2vecEvalNeg.argtypes = [ci, ci, ci, ci, ip, ip, fp, fp, cd, ci]
@@ -80,6 +82,12 @@ class CPUMACH:
     def word2vecNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, nthreads):
         _load().oracle_word2vecNeg(nrows, ncols, nwa, nwb, _i(WA), _i(WB), _f(A), _f(B),
                                    lrate, vexp, nthreads)
+
+    @staticmethod
+    def word2vecNegFilt(nrows, ncols, nwords, nwa, nwb, WA, WB, A, B, lrate, vexp, nthreads):
+        """CPU statement of the reference's GPU-only filtered negative pass (CUMACH.java:94)."""
+        _load().oracle_word2vecNegFilt(nrows, ncols, nwords, nwa, nwb, _i(WA), _i(WB), _f(A),
+                                       _f(B), lrate, vexp, nthreads)
 
     @staticmethod
     def word2vecEvalPos(nrows, ncols, skip, W, LB, UB, A, B, nthreads, floor=C_FLOOR):

@@ -10,6 +10,9 @@
  *   oracle_word2vecNeg      <- :186-264
  *   oracle_word2vecEvalPos  <- :368-427
  *   oracle_word2vecEvalNeg  <- :429-483
+ *   oracle_word2vecNegFilt  <- the same arithmetic as word2vecNeg under the id filter of the
+ *                              reference's GPU-only __word2vecNegFilt (jni/src/DNN127.cu:690-711):
+ *                              a word id >= nwords drops every pair it takes part in
  * with the JNI array pinning replaced by plain pointers.  Arithmetic order is
  * kept (fp32 multiply then add in ascending row order, exp/pow/log in double,
  * B updated inside the window loop, A after it) so that a single-threaded run
@@ -136,6 +139,31 @@ void oracle_word2vecNeg(int nrows, int ncols, int nwa, int nwb, const int *WA, c
     free(dbb);
     free(daa);
   }
+}
+
+void oracle_word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, const int *WA,
+                            const int *WB, float *A, float *B, float lrate, float vexp,
+                            int nthreads) {
+  /* Groups are rebuilt without the filtered ids and handed to the plain routine one at a time:
+   * dropping an id removes exactly the dot products and updates it would have taken part in. */
+  int i, j, k;
+  int *wa = (int *)malloc((size_t)(nwa > 0 ? nwa : 1) * sizeof(int));
+  int *wb = (int *)malloc((size_t)(nwb > 0 ? nwb : 1) * sizeof(int));
+  (void)nthreads;
+  for (i = 0; i < ncols; i++) {
+    int na = 0, nb = 0;
+    for (j = 0; j < nwa; j++) {
+      int id = WA[j + (int64_t)i * nwa];
+      if (id >= 0 && id < nwords) wa[na++] = id;
+    }
+    for (k = 0; k < nwb; k++) {
+      int id = WB[k + (int64_t)i * nwb];
+      if (id >= 0 && id < nwords) wb[nb++] = id;
+    }
+    if (na > 0 && nb > 0) oracle_word2vecNeg(nrows, 1, na, nb, wa, wb, A, B, lrate, vexp, 1);
+  }
+  free(wb);
+  free(wa);
 }
 
 double oracle_word2vecEvalPos(int nrows, int ncols, int skip, const int *W, const int *LB,

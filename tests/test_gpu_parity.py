@@ -300,6 +300,25 @@ def test_empty_and_rejected_arguments(gpu):
     assert CUMACH.word2vecEvalPos(d, 4, 5, I, I, I, A, B, ret) == 0
 
 
+@pytest.mark.parametrize("d,nwa,nwb", [(300, 5, 5), (100, 10, 5), (64, 5, 1)])
+def test_neg_filt_matches_oracle(gpu, oracle, d, nwa, nwb):
+    """word2vecNegFilt (CUMACH.java:94): tables hold nwords columns, larger ids are skipped."""
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(d + nwa)
+    V, G, nwords = 9000, 400, 6000
+    A, B = rand_tables(rng, V, d, 0.4 / math.sqrt(d) ** 0.5)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    Ao, Bo = A[:nwords].copy(), B[:nwords].copy()
+    oracle.word2vecNegFilt(d, G, nwords, nwa, nwb, WA, WB, Ao, Bo, 0.025, 0.5, 1)
+    Ad, Bd = dev(torch, A[:nwords]), dev(torch, B[:nwords])     # only nwords columns exist
+    err = CUMACH.word2vecNegFilt(d, G, nwords, nwa, nwb, dev(torch, WA), dev(torch, WB), Ad, Bd,
+                                 0.025, 0.5)
+    assert err == 0
+    assert np.abs(Ad.cpu().numpy() - Ao).max() <= UPDATE_ATOL
+    assert np.abs(Bd.cpu().numpy() - Bo).max() <= UPDATE_ATOL
+    assert np.abs(Ao - A[:nwords]).max() > 10 * UPDATE_ATOL
+
+
 def test_negative_ids_in_groups_are_skipped(gpu, oracle):
     """The reference reads WA/WB unchecked; the library skips pairs with a negative id."""
     rng = np.random.default_rng(31)

@@ -183,6 +183,34 @@ def test_neg_update_closed_form(oracle, vexp, d, nwa, nwb):
     assert np.abs(A2 - A).max() > 1e-4 and np.abs(B2 - B).max() > 1e-4
 
 
+def test_neg_filt_drops_pairs_with_filtered_ids(oracle):
+    """word2vecNegFilt: ids >= nwords take no part (DNN127.cu:690-711).  On a collision-free
+    minibatch the result is the closed form over the surviving ids of each group."""
+    rng = np.random.default_rng(14)
+    d, V, G, nwa, nwb, nwords = 16, 3000, 60, 5, 4, 2000
+    A, B = rand_tables(rng, V, d, 0.3)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    assert (WA >= nwords).any() and (WB >= nwords).any()
+    A2, B2 = A.copy(), B.copy()
+    oracle.word2vecNegFilt(d, G, nwords, nwa, nwb, WA, WB, A2, B2, 0.05, 0.5, 1)
+    Aw, Bw = A.astype(np.float64), B.astype(np.float64)
+    for g in range(G):
+        wa = WA[g * nwa:(g + 1) * nwa]
+        wb = WB[g * nwb:(g + 1) * nwb]
+        wa, wb = wa[wa < nwords], wb[wb < nwords]
+        if len(wa) and len(wb):
+            Ag, Bg = cf.neg_update(len(wa), len(wb), wa, wb, A, B, 0.05, 0.5)
+            Aw[wa], Bw[wb] = Ag[wa], Bg[wb]
+    np.testing.assert_allclose(A2, Aw, rtol=0, atol=2e-4)
+    np.testing.assert_allclose(B2, Bw, rtol=0, atol=2e-4)
+    assert np.array_equal(A2[nwords:], A[nwords:]) and np.array_equal(B2[nwords:], B[nwords:])
+    # with nwords beyond every id it is word2vecNeg
+    A3, B3, A4, B4 = A.copy(), B.copy(), A.copy(), B.copy()
+    oracle.word2vecNegFilt(d, G, V, nwa, nwb, WA, WB, A3, B3, 0.05, 0.5, 1)
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, A4, B4, 0.05, 0.5, 1)
+    assert np.array_equal(A3, A4) and np.array_equal(B3, B4)
+
+
 def test_first_minibatch_identity(oracle):
     """A == 0 (the model's start, Word2Vec.scala:117): dB = 0 and dA = ascale*lr*0.5*sum(B_ctx)."""
     rng = np.random.default_rng(5)
