@@ -60,6 +60,8 @@ SYMBOLS = {
     "w2v_memcpy_h2d": (_I, [_P, _P, _SZ]),
     "w2v_memcpy_d2h": (_I, [_P, _P, _SZ]),
     "w2v_memset": (_I, [_P, _I, _SZ]),
+    "w2v_wordmats": (_I, [_I, _P, _I, _I, _I, _I, _I, _F, _F, ctypes.c_ulonglong, ctypes.c_uint,
+                          _P, _P, _P, _P, _P, _P, ctypes.POINTER(_I)]),
     "w2v_timer_create": (_I, [ctypes.POINTER(_P)]),
     "w2v_timer_destroy": (_I, [_P]),
     "w2v_timer_start": (_I, [_P]),
@@ -188,6 +190,17 @@ class CUMACH:
     def word2vecEvalNegAsync(nrows, ncols, nwa, nwb, WA, WB, A, B, retVal):
         return load_library().word2vecEvalNegAsync(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB),
                                                    _ptr(A), _ptr(B), _ptr(retVal))
+
+
+def wordmats(n, mats, iflip, vocab, nskip, nneg, nreuse, wsample_lnv, wexpt, seed, call, words,
+             lb, ub, negs, ctx, counts):
+    """w2v_wordmats on device buffers; returns (number of valid pairs, number of groups)."""
+    host = (ctypes.c_int * 2)()
+    err = load_library().w2v_wordmats(n, _ptr(mats), int(bool(iflip)), vocab, nskip, nneg, nreuse,
+                                      wsample_lnv, wexpt, seed, call, _ptr(words), _ptr(lb),
+                                      _ptr(ub), _ptr(negs), _ptr(ctx), _ptr(counts), host)
+    check(err, "w2v_wordmats")
+    return int(host[0]), int(host[1])
 
 
 class Timer:

@@ -15,17 +15,19 @@ What is mirrored (src/main/scala/BIDMach/networks/Word2Vec.scala of the referenc
                   (istep - 1) % evalStep == 0, and so is the last one of a pass
                   (Learner.scala:187-222, evalStep default 11 at :1064)
 
-The arithmetic runs in the HIP library through bidmach_amd.cumach.CUMACH; this module only
-prepares index arrays (numpy, on the host, like the reference's CPU branch `getnegs`) and owns the
-device buffers (torch tensors: plumbing).  Random draws come from numpy, not from BIDMat, so a run
-reproduces the reference's distributions and array contracts, not its random stream.
+The arithmetic runs in the HIP library through bidmach_amd.cumach.CUMACH.  The index arrays are
+prepared either on the device (w2v_wordmats, the counterpart of the reference's GPU branch of
+wordMats, :241-270; the default on a GPU) or with numpy on the host (like the reference's CPU
+branch `getnegs`, :280-364); this module owns the device buffers (torch tensors: plumbing).
+Random draws come from numpy or from the library's counter-based generator, not from BIDMat, so
+a run reproduces the reference's distributions and array contracts, not its random stream.
 """
 import math
 
 import numpy as np
 
 from . import corpus
-from .cumach import CUMACH, check
+from .cumach import CUMACH, check, wordmats as _device_wordmats
 
 
 class Options:
@@ -48,6 +50,7 @@ class Options:
         self.batchSize = 100000
         self.evalStep = 11
         self.seed = 0
+        self.deviceWordMats = True   # build the index arrays on the GPU when the model is on one
         for k, v in kw.items():
             if not hasattr(self, k):
                 raise AttributeError("unknown Word2Vec option %r" % k)
@@ -63,6 +66,8 @@ class Word2Vec:
         self.ncols = None
         self.rng = np.random.Generator(np.random.PCG64(self.opts.seed))
         self._ret = None
+        self._call = 0
+        self._wm = None
 
     # ---- Word2Vec.init ------------------------------------------------------------------
     def init(self, ncols=None, modelmats=None):
@@ -122,6 +127,36 @@ class Word2Vec:
         import torch
         return torch.from_numpy(np.ascontiguousarray(x)).to(self.device)
 
+    # ---- Word2Vec.wordMats (device branch) ----------------------------------------------
+    def wordMatsDevice(self, mats):
+        """Same outputs as wordMats, as device tensors, built by the library on the GPU."""
+        import torch
+        o = self.opts
+        wordsens = np.asarray(mats)
+        n = wordsens.shape[1]
+        cap = 2 * o.nskip * n
+        if self._wm is None or self._wm["n"] != n:
+            def ibuf(k):
+                return torch.empty(max(k, 1), dtype=torch.int32, device=self.device)
+            self._wm = dict(n=n, words=ibuf(n), lb=ibuf(n), ub=ibuf(n), ctx=ibuf(cap),
+                            negs=ibuf(o.nneg * (cap // o.nreuse + 1)), counts=ibuf(2))
+        b = self._wm
+        # the data source's 2 x n matrix, column-major: (word, sentence) pairs interleaved
+        dmats = torch.from_numpy(np.ascontiguousarray(wordsens.T.astype(np.int32))).to(self.device)
+        self._call += 1
+        npairs, ngroups = _device_wordmats(n, dmats, o.iflip, o.vocabSize, o.nskip, o.nneg,
+                                           o.nreuse, float(np.float32(self.salpha)), o.wexpt,
+                                           o.seed, self._call, b["words"], b["lb"], b["ub"],
+                                           b["negs"], b["ctx"], b["counts"])
+        return (b["words"], b["lb"], b["ub"], b["negs"][:ngroups * o.nneg],
+                b["ctx"][:ngroups * o.nreuse])
+
+    def _index_arrays(self, mats):
+        """(words, lb, ub, trandwords, contextwords) on the model's device."""
+        if self.opts.deviceWordMats and str(self.device).startswith("cuda"):
+            return self.wordMatsDevice(mats)
+        return tuple(self._dev(x) for x in self.wordMats(mats))
+
     # ---- the four dispatchers (Word2Vec.scala:366-402, 469-523) --------------------------
     def procPositives(self, nskip, words, lb, ub, model1, model2, lrate, vexp):
         nrows = model1.shape[1]
@@ -156,27 +191,25 @@ class Word2Vec:
             self.firstPos = pos
         nsteps = float(pos) / float(self.firstPos)
         lrate = float(o.lrate) * math.pow(nsteps, -o.texp)
-        words, lb, ub, trandwords, goodwords = self.wordMats(mats)
+        words, lb, ub, trandwords, goodwords = self._index_arrays(mats)
         lrpos = lrate
         lrneg = lrpos if o.eqPosNeg else lrpos / o.nneg
-        dw, dlb, dub = self._dev(words), self._dev(lb), self._dev(ub)
-        self.procPositives(o.nskip, dw, dlb, dub, self.modelmats[1], self.modelmats[0], lrpos,
+        self.procPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0], lrpos,
                            o.vexp)
         if goodwords.shape[0] > 0:
-            self.procNegatives(o.nneg, o.nreuse, self._dev(trandwords), self._dev(goodwords),
-                               self.modelmats[1], self.modelmats[0], lrneg, o.vexp)
+            self.procNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
+                               self.modelmats[0], lrneg, o.vexp)
 
     def evalbatch(self, mats, ipass, pos):
         o = self.opts
         if np.asarray(mats).shape[1] != self.ncols:
             return 0.0                                          # row(0) (:211)
-        words, lb, ub, trandwords, goodwords = self.wordMats(mats)
+        words, lb, ub, trandwords, goodwords = self._index_arrays(mats)
         if goodwords.shape[0] == 0:
             return 0.0
-        epos = self.evalPositives(o.nskip, self._dev(words), self._dev(lb), self._dev(ub),
-                                  self.modelmats[1], self.modelmats[0])
-        eneg = self.evalNegatives(o.nneg, o.nreuse, self._dev(trandwords), self._dev(goodwords),
-                                  self.modelmats[1], self.modelmats[0])
+        epos = self.evalPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0])
+        eneg = self.evalNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
+                                  self.modelmats[0])
         return (epos + eneg / (1 if o.eqPosNeg else o.nneg)) / goodwords.shape[0]
 
     # ---- Learner.nextPass, reduced to what Word2Vec uses (no updater, no mixins) ---------

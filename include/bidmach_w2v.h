@@ -114,6 +114,24 @@ int w2v_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes);
 int w2v_memcpy_d2h(void *host_dst, const void *dev_src, size_t bytes);
 int w2v_memset(void *dev_ptr, int value, size_t bytes);
 
+/* Minibatch preprocessing on the device: the step before the operators, what
+ * Word2Vec.wordMats does (Word2Vec.scala:214-364; its GPU branch :241-270).  No counterpart in
+ * the reference's native library (there it is a chain of BIDMat matrix operations).
+ *   mats        device, the 2 x n IMat of the data source, column-major: mats[2*i] word id,
+ *               mats[2*i+1] sentence id of token i (swapped when iflip != 0)
+ *   wsample_lnv wsample * ln(vocabSize) (Word2Vec.scala:150); wexpt the negative-sampling
+ *               exponent (0.75)
+ *   seed, call  key of the counter-based random generator; pass a new `call` for every minibatch
+ *   words, lb, ub   device int[n] outputs: the W, LB, UB arguments of word2vecPos
+ *   negs        device int[nneg * G] output (capacity nneg * ceil(2*nskip*n / nreuse)): WA
+ *   ctx         device int[2*nskip*n] output; its first nreuse*G entries are WB
+ *   counts_dev  device int[2]: {number of valid pairs, G}; counts_host (may be NULL) gets a copy
+ * Blocking (it reads the pair count back to size the rest of the work). */
+int w2v_wordmats(int n, const int *mats, int iflip, int vocab, int nskip, int nneg, int nreuse,
+                 float wsample_lnv, float wexpt, unsigned long long seed, unsigned call,
+                 int *words, int *lb, int *ub, int *negs, int *ctx, int *counts_dev,
+                 int *counts_host);
+
 /* Event-pair timers on the calling thread's launch stream. */
 int w2v_timer_create(void **timer);
 int w2v_timer_destroy(void *timer);

@@ -22,7 +22,8 @@ def make_stream(n, vocab, seed=3):
 def test_dobatch_and_evalbatch_match_cpu_twin(oracle):
     import torch
     assert torch.cuda.is_available()
-    o = dict(vocabSize=4000, dim=64, batchSize=8000, lrate=0.005, vexp=0.5, texp=0.5, seed=11)
+    o = dict(vocabSize=4000, dim=64, batchSize=8000, lrate=0.005, vexp=0.5, texp=0.5, seed=11,
+             deviceWordMats=False)     # host-built index arrays, so the CPU twin sees the same ones
     gpu = Word2Vec(Options(**o), device="cuda:0")
     twin = Word2Vec(Options(**o), device="cpu")     # same seed: same init, same wordMats draws
     gpu.init()
@@ -69,6 +70,28 @@ def test_train_loop_scores_held_out_minibatches():
     scores = [r[1] for r in res]
     assert all(np.isfinite(s) and s < 0 for s in scores)
     assert scores[-1] > scores[0]            # the log-likelihood per context word went up
+
+
+def test_device_wordmats_path_matches_oracle_step(oracle):
+    """dobatch with index arrays built on the device: the arrays are read back and the same step
+    is replayed with the CPU oracle."""
+    o = Options(vocabSize=4000, dim=64, batchSize=6000, lrate=0.005, vexp=0.5, seed=3)
+    m = Word2Vec(o)
+    m.init()
+    m0 = m.modelmats[0].cpu().numpy().copy()
+    m1 = m.modelmats[1].cpu().numpy().copy()
+    mats = make_stream(6000, 4000, seed=21)
+    m.dobatch(mats, 0, 6000)
+    b = m._wm
+    npairs, G = b["counts"].cpu().tolist()
+    words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
+    negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
+    ctx = b["ctx"].cpu().numpy()[:G * o.nreuse].copy()
+    assert G > 100 and npairs // o.nreuse == G
+    oracle.word2vecPos(64, 6000, o.nskip, words, lb, ub, m1, m0, 0.005, 0.5, 1)
+    oracle.word2vecNeg(64, G, o.nneg, o.nreuse, negs, ctx, m1, m0, 0.005 / o.nneg, 0.5, 1)
+    assert np.abs(m.modelmats[0].cpu().numpy() - m0).max() < 2e-3
+    assert np.abs(m.modelmats[1].cpu().numpy() - m1).max() < 2e-3
 
 
 def test_odd_sized_minibatch_is_skipped():
