@@ -65,6 +65,7 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
     err = hipMalloc(reinterpret_cast<void**>(&p), 2 * bytes);
     if (err != hipSuccess) return err;
     err = hipMemsetAsync(p, 0, 2 * bytes, ts.stream);
+    if (err == hipSuccess) err = hipStreamSynchronize(ts.stream);  // the stream may change later
     if (err != hipSuccess) {
       (void)hipFree(p);
       return err;

@@ -115,3 +115,60 @@ def test_heldout_loss_raw_stream_stays_finite_and_close(oracle):
     assert np.isfinite(gpu) and np.isfinite(gpu8)
     assert abs(gpu - cpu_seq) <= 0.15 * cpu_seq, (gpu, cpu_seq)
     assert abs(gpu8 - cpu_seq) <= 0.15 * cpu_seq, (gpu8, cpu_seq)
+
+
+def test_headline_shape_subsampled_loss_and_full_size_eval(oracle):
+    """The headline shape itself (vocab 1M, dim 300, 1M-token minibatches, window 5, 5 negatives),
+    with the reference caller's default subsampling: 12 minibatches on the GPU and on the CPU
+    oracle (16 Hogwild threads, as the reference would run it), then the held-out score of both.
+    Also a full-size forward-only check: the GPU scores the CPU-trained tables and must agree
+    with the oracle's sums to 1e-5."""
+    import torch
+    from bidmach_amd.cumach import CUMACH, check
+    Vh, Dh, Nh, K = 1_000_000, 300, 1_000_000, 12
+    zc = corpus.zipf_cdf(Vh, 1.0)
+    nc = corpus.unigram_pow_cdf(Vh, 1.0, 0.75)
+
+    def mb(i):
+        W = corpus.zipf_stream(Nh, Vh, 1.0, seed=1234 + i, cdf=zc)
+        rng = np.random.Generator(np.random.PCG64(99 + i))
+        W = corpus.subsample(W, Vh, 1.0e-4, rng)
+        LB, UB = corpus.window_bounds(Nh, SKIP, rng)
+        WA, WB, G = corpus.negative_groups(W, LB, UB, NNEG, NREUSE, rng, neg_cdf=nc)
+        return W, LB, UB, WA, WB, G
+
+    def lr(i):
+        return max(LR0 * (1.0 - i / K), LR0 * 1e-4)
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    mbs = [mb(i) for i in range(K + 1)]
+    B, A = corpus.init_tables(Vh, Dh, 42)
+    Bd, Ad = dev(B), dev(A)
+    for i in range(K):
+        W, LB, UB, WA, WB, G = mbs[i]
+        oracle.word2vecPos(Dh, Nh, SKIP, W, LB, UB, A, B, lr(i), 0.0, 16)
+        oracle.word2vecNeg(Dh, G, NNEG, NREUSE, WA, WB, A, B, lr(i) / NNEG, 0.0, 16)
+        check(CUMACH.word2vecPos(Dh, Nh, SKIP, dev(W), dev(LB), dev(UB), Ad, Bd, lr(i), 0.0), "pos")
+        check(CUMACH.word2vecNeg(Dh, G, NNEG, NREUSE, dev(WA), dev(WB), Ad, Bd, lr(i) / NNEG, 0.0),
+              "neg")
+    W, LB, UB, WA, WB, G = mbs[K]
+    epos = oracle.word2vecEvalPos(Dh, Nh, SKIP, W, LB, UB, A, B, 16)
+    eneg = oracle.word2vecEvalNeg(Dh, G, NNEG, NREUSE, WA, WB, A, B, 16)
+    cpu = -(epos + eneg / NNEG) / (G * NREUSE)
+    dW, dLB, dUB, dWA, dWB = dev(W), dev(LB), dev(UB), dev(WA), dev(WB)
+    ret = torch.zeros(4, dtype=torch.float64, device="cuda")
+    check(CUMACH.word2vecEvalPosF64(Dh, Nh, SKIP, dW, dLB, dUB, Ad, Bd, ret[0:1]), "epos")
+    check(CUMACH.word2vecEvalNegF64(Dh, G, NNEG, NREUSE, dWA, dWB, Ad, Bd, ret[1:2]), "eneg")
+    # full-size forward-only parity on identical (CPU-trained) tables
+    Ac, Bc = dev(A), dev(B)
+    check(CUMACH.word2vecEvalPosF64(Dh, Nh, SKIP, dW, dLB, dUB, Ac, Bc, ret[2:3]), "epos")
+    check(CUMACH.word2vecEvalNegF64(Dh, G, NNEG, NREUSE, dWA, dWB, Ac, Bc, ret[3:4]), "eneg")
+    r = ret.cpu().numpy()
+    gpu = -(r[0] + r[1] / NNEG) / (G * NREUSE)
+    print("\nheadline shape, subsampled: held-out loss cpu(16 threads) %.5f gpu %.5f rel %+.3f%%"
+          % (cpu, gpu, 100.0 * (gpu / cpu - 1.0)))
+    assert r[2] == pytest.approx(epos, rel=1e-5)
+    assert r[3] == pytest.approx(eneg, rel=1e-5)
+    assert abs(gpu - cpu) <= 0.005 * cpu, (gpu, cpu)
