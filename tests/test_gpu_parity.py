@@ -348,6 +348,55 @@ def test_negative_ids_in_groups_are_skipped(gpu, oracle):
 # Colliding (Zipf) minibatches: statistical agreement
 # ---------------------------------------------------------------------------------------------
 
+def test_column_offsets_beyond_2_to_31_elements(gpu, oracle):
+    """Tables of 7.3 M x 300 floats: the columns used here start beyond element 2^31, where the
+    reference's 32-bit `nrows * id` offset (BIDMach_CPUMACH.c:31) would overflow.  With vexp = 0
+    the result does not depend on the id values, so the oracle runs on a compact copy of the
+    touched columns with the ids renumbered."""
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(91)
+    d, V, skip, nwa, nwb = 300, 7_300_000, 5, 5, 5
+    first = (1 << 31) // d + 1                      # first id whose column starts past 2^31
+    assert first + 5000 < V
+    n_ids = 4000
+    big = (first + rng.permutation(V - first)[:n_ids]).astype(np.int64)
+    assert (big * d > (1 << 31)).all()
+    Ac = (rng.standard_normal((n_ids, d)) * 0.1).astype(np.float32)   # compact tables
+    Bc = (rng.standard_normal((n_ids, d)) * 0.1).astype(np.float32)
+    A = torch.zeros((V, d), dtype=torch.float32, device="cuda")
+    B = torch.zeros((V, d), dtype=torch.float32, device="cuda")
+    idx = torch.from_numpy(big).cuda()
+    A[idx] = torch.from_numpy(Ac).cuda()
+    B[idx] = torch.from_numpy(Bc).cuda()
+    # positive pass: 100 centres with full windows over compact ids 0..1099
+    Wc, LB, UB = corpus.collision_free_pos(100, skip, 1100, np.random.default_rng(1))
+    # negative pass: 200 groups over compact ids 1100..3099
+    WAc, WBc = corpus.collision_free_neg(200, nwa, nwb, 2000, np.random.default_rng(2))
+    WAc, WBc = WAc + 1100, WBc + 1100
+    Ao, Bo = Ac.copy(), Bc.copy()
+    oracle.word2vecPos(d, Wc.shape[0], skip, Wc, LB, UB, Ao, Bo, 0.025, 0.0, 1)
+    oracle.word2vecNeg(d, 200, nwa, nwb, WAc, WBc, Ao, Bo, 0.005, 0.0, 1)
+    tobig = big.astype(np.int32)
+    assert CUMACH.word2vecPos(d, Wc.shape[0], skip, dev(torch, tobig[Wc]), dev(torch, LB),
+                              dev(torch, UB), A, B, 0.025, 0.0) == 0
+    assert CUMACH.word2vecNeg(d, 200, nwa, nwb, dev(torch, tobig[WAc]), dev(torch, tobig[WBc]), A,
+                              B, 0.005, 0.0) == 0
+    assert np.abs(A[idx].cpu().numpy() - Ao).max() <= UPDATE_ATOL
+    assert np.abs(B[idx].cpu().numpy() - Bo).max() <= UPDATE_ATOL
+    assert np.abs(Ao - Ac).max() > 10 * UPDATE_ATOL
+    # nothing else was touched
+    A[idx] = 0
+    B[idx] = 0
+    assert float(A.abs().max().item()) == 0.0 and float(B.abs().max().item()) == 0.0
+    ret = torch.zeros(1, dtype=torch.float64, device="cuda")
+    A[idx] = torch.from_numpy(Ao).cuda()
+    B[idx] = torch.from_numpy(Bo).cuda()
+    assert CUMACH.word2vecEvalPosF64(d, Wc.shape[0], skip, dev(torch, tobig[Wc]), dev(torch, LB),
+                                     dev(torch, UB), A, B, ret) == 0
+    want = oracle.word2vecEvalPos(d, Wc.shape[0], skip, Wc, LB, UB, Ao, Bo, 1)
+    assert float(ret.item()) == pytest.approx(want, rel=EVAL_RTOL)
+
+
 def _rows_close(got, want, rtol, atol):
     err = np.abs(got - want).max(axis=1)
     lim = rtol * np.abs(want).max(axis=1) + atol
