@@ -61,7 +61,7 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
                            const int* WA, const int* WB, const float* A, const float* B,
                            double floorv, double* partials, float* Retval32, double* Retval64);
 
-hipError_t launch_finalize(hipStream_t stream, const double* partials, int64_t n, float* Retval32,
+hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, float* Retval32,
                            double* Retval64);
 
 // Largest nrows / nwb the register-resident kernels take; beyond them the calls fail with

@@ -365,22 +365,43 @@ hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, in
   return hipSuccess;
 }
 
-// Folds the per-block partial sums in a fixed order (thread t takes t, t+256, ...; then a
-// fixed LDS tree), so the result does not depend on block scheduling.
-__global__ void __launch_bounds__(kBlock)
-finalize_kernel(const double* __restrict__ partials, int64_t n, float* Retval32, double* Retval64) {
-  __shared__ double s[kBlock];
-  double t = 0.0;
-  for (int64_t k = threadIdx.x; k < n; k += kBlock) t += partials[k];
+// Sum of the block's 256 per-thread values by a fixed LDS tree; the result is valid in thread 0.
+__device__ __forceinline__ double block_tree_sum(double t, double* s) {
   s[threadIdx.x] = t;
   __syncthreads();
   for (int w = kBlock / 2; w > 0; w >>= 1) {
     if ((int)threadIdx.x < w) s[threadIdx.x] += s[threadIdx.x + w];
     __syncthreads();
   }
+  return s[0];
+}
+
+// First stage of the fold for long partial arrays: block b sums its slice [b*len, (b+1)*len) in a
+// fixed order and leaves the sum in the slice's first element (it has read the whole slice before
+// it writes, and no other block touches the slice).
+__global__ void __launch_bounds__(kBlock)
+finalize_slices_kernel(double* __restrict__ partials, int64_t n, int64_t len) {
+  __shared__ double s[kBlock];
+  const int64_t base = (int64_t)blockIdx.x * len;
+  const int64_t end = base + len < n ? base + len : n;
+  double t = 0.0;
+  for (int64_t k = base + threadIdx.x; k < end; k += kBlock) t += partials[k];
+  const double total = block_tree_sum(t, s);
+  if (threadIdx.x == 0) partials[base] = total;
+}
+
+// Folds partials[0], partials[stride], ... (n of them) in a fixed order (thread t takes t, t+256,
+// ...; then a fixed LDS tree), so the result does not depend on block scheduling.
+__global__ void __launch_bounds__(kBlock)
+finalize_kernel(const double* __restrict__ partials, int64_t n, int64_t stride, float* Retval32,
+                double* Retval64) {
+  __shared__ double s[kBlock];
+  double t = 0.0;
+  for (int64_t k = threadIdx.x; k < n; k += kBlock) t += partials[k * stride];
+  const double total = block_tree_sum(t, s);
   if (threadIdx.x == 0) {
-    if (Retval32 != nullptr) Retval32[0] += (float)s[0];
-    if (Retval64 != nullptr) Retval64[0] += s[0];
+    if (Retval32 != nullptr) Retval32[0] += (float)total;
+    if (Retval64 != nullptr) Retval64[0] += total;
   }
 }
 
@@ -458,10 +479,22 @@ hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const
 #undef CALL
 }
 
-hipError_t launch_finalize(hipStream_t stream, const double* partials, int64_t n, float* Retval32,
+hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, float* Retval32,
                            double* Retval64) {
-  hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kBlock), 0, stream, partials, n, Retval32,
-                     Retval64);
+  // Long arrays are first cut into at most 1024 slices summed by one block each.
+  constexpr int64_t kSliceMin = 256;
+  int64_t stride = 1;
+  if (n > 4 * kSliceMin) {
+    int64_t len = (n + 1023) / 1024;
+    if (len < kSliceMin) len = kSliceMin;
+    const int64_t slices = (n + len - 1) / len;
+    hipLaunchKernelGGL(finalize_slices_kernel, dim3((unsigned)slices), dim3(kBlock), 0, stream,
+                       partials, n, len);
+    stride = len;
+    n = slices;
+  }
+  hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kBlock), 0, stream, partials, n, stride,
+                     Retval32, Retval64);
   return hipGetLastError();
 }
 
