@@ -145,6 +145,93 @@ int eval_neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, floa
                 sync);
 }
 
+// Checks the slicing arguments and gathers the model-matrix pointers the kernels may touch.
+// With dualMode the first pair of MM belongs to the device half of a dual-mode model
+// (Word2Vec.scala:118-131 of the reference) and the parts start at MM[2].
+bool slice_map(float** MM, int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+               int doHead, w2v::SliceMap* out) {
+  const int offset = dualMode ? 1 : 0;
+  if (!MM || nmats < 2 * (offset + 1) || (nmats & 1) || nslices < 1 || islice < 0 ||
+      islice >= nslices || maxCols < 1 || nHead < 0 || doHead < 0)
+    return false;
+  const int nparts = nmats / 2 - offset;
+  if (nparts > w2v::max_slice_parts()) return false;
+  w2v::SliceMap m{};
+  for (int k = 0; k < 2 * nparts; ++k) {
+    m.mats[k] = MM[2 * offset + k];
+    if (m.mats[k] == nullptr) return false;
+  }
+  m.nparts = nparts;
+  m.islice = islice;
+  m.nslices = nslices;
+  m.nhead = nHead;
+  m.maxcols = maxCols;
+  m.dohead = doHead;
+  *out = m;
+  return true;
+}
+
+int pos_slice_impl(int nrows, int ncols, int* W, int* LB, int* UB, float** MM, int nmats,
+                   float lrate, float vexp, int islice, int nslices, int maxCols, int nHead,
+                   int dualMode, int doHead) {
+  w2v::SliceMap m;
+  if (bad_common(nrows, ncols) ||
+      !slice_map(MM, nmats, islice, nslices, maxCols, nHead, dualMode, doHead, &m))
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_slice_pos(t_state.stream, nrows, ncols, W, LB, UB, m, lrate, vexp),
+                true);
+}
+
+int neg_slice_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float** MM, int nmats,
+                   float lrate, float vexp, int islice, int nslices, int maxCols, int nHead,
+                   int dualMode, int doHead) {
+  w2v::SliceMap m;
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() ||
+      !slice_map(MM, nmats, islice, nslices, maxCols, nHead, dualMode, doHead, &m))
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_slice_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate,
+                                      vexp),
+                true);
+}
+
+int eval_pos_slice_impl(int nrows, int ncols, int* W, int* LB, int* UB, float** MM, int nmats,
+                        int islice, int nslices, int maxCols, int nHead, int dualMode,
+                        double* Retval) {
+  w2v::SliceMap m;
+  if (bad_common(nrows, ncols) || !Retval ||
+      !slice_map(MM, nmats, islice, nslices, maxCols, nHead, dualMode, 0, &m))
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB) return (int)hipErrorInvalidValue;
+  double* partials = nullptr;
+  hipError_t err = eval_scratch(w2v::slice_eval_partials_needed(), &partials);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_slice_eval_pos(t_state.stream, nrows, ncols, W, LB, UB, m,
+                                           g_eval_floor.load(), partials, nullptr, Retval),
+                true);
+}
+
+int eval_neg_slice_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float** MM,
+                        int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+                        double* Retval) {
+  w2v::SliceMap m;
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || !Retval ||
+      !slice_map(MM, nmats, islice, nslices, maxCols, nHead, dualMode, 0, &m))
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB) return (int)hipErrorInvalidValue;
+  double* partials = nullptr;
+  hipError_t err = eval_scratch(w2v::slice_eval_partials_needed(), &partials);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_slice_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, m,
+                                           g_eval_floor.load(), partials, nullptr, Retval),
+                true);
+}
+
 struct Timer {
   hipEvent_t start;
   hipEvent_t stop;
@@ -168,6 +255,38 @@ int word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, int* WA,
                     float* B, float lrate, float vexp) {
   return neg_impl(nrows, ncols, nwords, nwa, nwb, WA, WB, A, B, lrate, vexp, true);
 }
+
+int word2vecPosSlice(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float** MM,
+                     int nmats, float lrate, float vexp, int islice, int nslices, int maxCols,
+                     int nHead, int dualMode, int doHead) {
+  (void)shift;
+  return pos_slice_impl(nrows, ncols, W, LB, UB, MM, nmats, lrate, vexp, islice, nslices, maxCols,
+                        nHead, dualMode, doHead);
+}
+
+int word2vecNegSlice(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float** MM,
+                     int nmats, float lrate, float vexp, int islice, int nslices, int maxCols,
+                     int nHead, int dualMode, int doHead) {
+  return neg_slice_impl(nrows, ncols, nwa, nwb, WA, WB, MM, nmats, lrate, vexp, islice, nslices,
+                        maxCols, nHead, dualMode, doHead);
+}
+
+int word2vecEvalPosSlice(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float** MM,
+                         int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+                         double* Retval) {
+  (void)shift;
+  return eval_pos_slice_impl(nrows, ncols, W, LB, UB, MM, nmats, islice, nslices, maxCols, nHead,
+                             dualMode, Retval);
+}
+
+int word2vecEvalNegSlice(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float** MM,
+                         int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+                         double* Retval) {
+  return eval_neg_slice_impl(nrows, ncols, nwa, nwb, WA, WB, MM, nmats, islice, nslices, maxCols,
+                             nHead, dualMode, Retval);
+}
+
+int w2v_max_slice_parts(void) { return w2v::max_slice_parts(); }
 
 int word2vecEvalPos(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
                     float* Retval) {

@@ -64,6 +64,35 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
 hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, float* Retval32,
                            double* Retval64);
 
+// A sliced, multi-part model as the kernels see it: part m has its B table at mats[2m] and its A
+// table at mats[2m+1], each of maxcols columns (the last part may be shorter).  Passed by value.
+constexpr int kMaxSliceParts = 32;
+struct SliceMap {
+  float* mats[2 * kMaxSliceParts];
+  int nparts;   // parts present; a word whose packed column falls beyond them is skipped
+  int islice;   // this worker
+  int nslices;  // workers the tail of the vocabulary is dealt to
+  int nhead;    // ids below this are resident on every worker
+  int maxcols;  // columns per part
+  int dohead;   // 0: head columns read-only, 1: written, 2: written and head-head pairs trained
+};
+
+int max_slice_parts();
+// Capacity the Eval launchers below need in `partials`.
+int64_t slice_eval_partials_needed();
+
+hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                            const int* UB, const SliceMap& m, float lrate, float vexp);
+hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                            const int* WA, const int* WB, const SliceMap& m, float lrate,
+                            float vexp);
+hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const int* W,
+                                 const int* LB, const int* UB, const SliceMap& m, double floorv,
+                                 double* partials, float* Retval32, double* Retval64);
+hipError_t launch_slice_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                 const int* WA, const int* WB, const SliceMap& m, double floorv,
+                                 double* partials, float* Retval32, double* Retval64);
+
 // Largest nrows / nwb the register-resident kernels take; beyond them the calls fail with
 // hipErrorInvalidValue.
 int max_rows();

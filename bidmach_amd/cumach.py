@@ -30,6 +30,7 @@ def lib_path():
 
 # name -> (restype, argtypes); every symbol include/bidmach_w2v.h declares.
 _I, _F, _D, _P, _SZ = ctypes.c_int, ctypes.c_float, ctypes.c_double, ctypes.c_void_p, ctypes.c_size_t
+_PP = ctypes.POINTER(ctypes.c_void_p)
 _POS = [_I, _I, _I, _P, _P, _P, _P, _P, _F, _F]
 _NEG = [_I, _I, _I, _I, _P, _P, _P, _P, _F, _F]
 _EPOS = [_I, _I, _I, _P, _P, _P, _P, _P, _P]
@@ -38,6 +39,11 @@ SYMBOLS = {
     "word2vecPos": (_I, _POS),
     "word2vecNeg": (_I, _NEG),
     "word2vecNegFilt": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P, _F, _F]),
+    "word2vecPosSlice": (_I, [_I, _I, _I, _P, _P, _P, _PP, _I, _F, _F, _I, _I, _I, _I, _I, _I]),
+    "word2vecNegSlice": (_I, [_I, _I, _I, _I, _P, _P, _PP, _I, _F, _F, _I, _I, _I, _I, _I, _I]),
+    "word2vecEvalPosSlice": (_I, [_I, _I, _I, _P, _P, _P, _PP, _I, _I, _I, _I, _I, _I, _P]),
+    "word2vecEvalNegSlice": (_I, [_I, _I, _I, _I, _P, _P, _PP, _I, _I, _I, _I, _I, _I, _P]),
+    "w2v_max_slice_parts": (_I, []),
     "word2vecEvalPos": (_I, _EPOS),
     "word2vecEvalNeg": (_I, _ENEG),
     "word2vecEvalPosF64": (_I, _EPOS),
@@ -120,6 +126,14 @@ def _ptr(x):
     raise TypeError("not a device pointer: %r" % type(x))
 
 
+def _ptr_array(mats):
+    """Host array of device addresses for a list of model matrices (a float** argument)."""
+    arr = (ctypes.c_void_p * len(mats))()
+    for k, m in enumerate(mats):
+        arr[k] = _ptr(m)
+    return arr
+
+
 def error_string(err):
     return load_library().w2v_error_string(int(err)).decode()
 
@@ -158,6 +172,37 @@ class CUMACH:
     def word2vecEvalNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, retVal):
         return load_library().word2vecEvalNeg(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB),
                                               _ptr(A), _ptr(B), _ptr(retVal))
+
+    # -- sliced, multi-part models: device counterparts of CPUMACH.java:14,19 and of the Scala
+    # -- forward twins (Word2Vec.scala:1007-1069, 1134-1200); MM is the list of model matrices
+
+    @staticmethod
+    def word2vecPosSlice(nrows, ncols, shift, W, LB, UB, MM, lrate, vexp, islice, nslices,
+                         maxCols, nHead, dualMode, doHead):
+        return load_library().word2vecPosSlice(
+            nrows, ncols, shift, _ptr(W), _ptr(LB), _ptr(UB), _ptr_array(MM), len(MM), lrate, vexp,
+            islice, nslices, maxCols, nHead, int(dualMode), doHead)
+
+    @staticmethod
+    def word2vecNegSlice(nrows, ncols, nwa, nwb, WA, WB, MM, lrate, vexp, islice, nslices,
+                         maxCols, nHead, dualMode, doHead):
+        return load_library().word2vecNegSlice(
+            nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB), _ptr_array(MM), len(MM), lrate, vexp,
+            islice, nslices, maxCols, nHead, int(dualMode), doHead)
+
+    @staticmethod
+    def word2vecEvalPosSlice(nrows, ncols, shift, W, LB, UB, MM, islice, nslices, maxCols, nHead,
+                             dualMode, retVal):
+        return load_library().word2vecEvalPosSlice(
+            nrows, ncols, shift, _ptr(W), _ptr(LB), _ptr(UB), _ptr_array(MM), len(MM), islice,
+            nslices, maxCols, nHead, int(dualMode), _ptr(retVal))
+
+    @staticmethod
+    def word2vecEvalNegSlice(nrows, ncols, nwa, nwb, WA, WB, MM, islice, nslices, maxCols, nHead,
+                             dualMode, retVal):
+        return load_library().word2vecEvalNegSlice(
+            nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB), _ptr_array(MM), len(MM), islice, nslices,
+            maxCols, nHead, int(dualMode), _ptr(retVal))
 
     # -- extensions of the library (no Java counterpart) ---------------------------------
 

@@ -11,6 +11,11 @@ What is mirrored (src/main/scala/BIDMach/networks/Word2Vec.scala of the referenc
   dobatch         learning-rate decay lrate * (pos/firstPos)**(-texp), then procPositives and
                   procNegatives with A = modelmats(1), B = modelmats(0) (:167-190, :366-402)
   evalbatch       (epos + eneg/nneg) / #context words (:192-212, :469-523)
+  sliced models   nSlices / iSlice / nHeadTerms / maxArraySize / dualMode / doHead: the packed,
+                  multi-part list of model matrices of :100-131 and the dispatch to the Slice
+                  operators when nSlices != 1 or the model needs more than one part (:178-187,
+                  :196-207).  The reference runs those on the CPU only; here every part is a
+                  device allocation and the library's device Slice operators are used.
   train           Learner.nextPass' loop: minibatch istep is scored instead of trained on when
                   (istep - 1) % evalStep == 0, and so is the last one of a pass
                   (Learner.scala:187-222, evalStep default 11 at :1064)
@@ -50,6 +55,12 @@ class Options:
         self.batchSize = 100000
         self.evalStep = 11
         self.seed = 0
+        self.maxArraySize = 2047 * 1024 * 1024
+        self.nHeadTerms = 0
+        self.nSlices = 1
+        self.iSlice = 0
+        self.dualMode = False
+        self.doHead = 1
         self.deviceWordMats = True   # build the index arrays on the GPU when the model is on one
         for k, v in kw.items():
             if not hasattr(self, k):
@@ -71,22 +82,41 @@ class Word2Vec:
 
     # ---- Word2Vec.init ------------------------------------------------------------------
     def init(self, ncols=None, modelmats=None):
+        """modelmats: optional host arrays in the layout of the reference's list, B table of part
+        m at 2m (+2 with a dual-mode list), A table at 2m+1; each (columns, dim) in C order."""
         import torch
         o = self.opts
         self.ncols = ncols if ncols is not None else o.batchSize
+        self.maxCols = o.maxArraySize // o.dim
+        # columns this worker holds: the head and its share of the tail (:106)
+        actual = o.nHeadTerms + 1 + (o.vocabSize - o.nHeadTerms - 1) // o.nSlices
+        self.nmmats = 1 + (actual - 1) // self.maxCols
+        self._dual = bool(o.dualMode) and self.nmmats > 1
         if modelmats is None:
-            m0 = (self.rng.random((o.vocabSize, o.dim), dtype=np.float32) - np.float32(0.5)) \
-                / np.float32(o.dim)
-            m1 = np.zeros((o.vocabSize, o.dim), dtype=np.float32)
-        else:
-            m0, m1 = modelmats
-        # (vocab, dim) C-order == dim x vocab column-major, the layout the operators take
-        self.modelmats = [torch.from_numpy(np.ascontiguousarray(m0)).to(self.device),
-                          torch.from_numpy(np.ascontiguousarray(m1)).to(self.device)]
+            def fresh(cols):
+                m0 = (self.rng.random((cols, o.dim), dtype=np.float32) - np.float32(0.5)) \
+                    / np.float32(o.dim)
+                return m0, np.zeros((cols, o.dim), dtype=np.float32)
+            if self.nmmats == 1:
+                modelmats = list(fresh(actual))
+            else:
+                modelmats = []
+                for i in range(self.nmmats):
+                    last = i == self.nmmats - 1
+                    modelmats += list(fresh(actual - i * self.maxCols if last else self.maxCols))
+                if self._dual:                         # the device copy of the first part (:128-131)
+                    modelmats = [modelmats[0].copy(), modelmats[1].copy()] + modelmats
+        # (columns, dim) C-order == dim x columns column-major, the layout the operators take
+        self.modelmats = [torch.from_numpy(np.ascontiguousarray(m)).to(self.device)
+                          for m in modelmats]
         self.expt = 1.0 / (1.0 - o.wexpt)
         self.salpha = o.wsample * math.log(o.vocabSize)
         self._ret = torch.zeros(2, dtype=torch.float32, device=self.device)
+        self._ret64 = torch.zeros(2, dtype=torch.float64, device=self.device)
         self.firstPos = -1
+
+    def _sliced(self):
+        return self.opts.nSlices != 1 or self.nmmats != 1
 
     # ---- Word2Vec.wordMats (host branch) ------------------------------------------------
     def wordMats(self, mats):
@@ -182,6 +212,35 @@ class Word2Vec:
                                      modela, modelb, self._ret[1:2]), "word2vecEvalNeg")
         return float(self._ret[1].item())
 
+    # ---- the Slice dispatchers (Word2Vec.scala:404-467, 491-534) ------------------------
+    def _slice_args(self):
+        o = self.opts
+        return (o.iSlice, o.nSlices, self.maxCols, o.nHeadTerms, self._dual)
+
+    def procPositivesSlice(self, nskip, words, lb, ub, modelmats, lrate, vexp):
+        check(CUMACH.word2vecPosSlice(self.opts.dim, words.shape[0], nskip, words, lb, ub,
+                                      modelmats, lrate, vexp, *self._slice_args(),
+                                      self.opts.doHead), "word2vecPosSlice")
+
+    def procNegativesSlice(self, nwa, nwb, wordsa, wordsb, modelmats, lrate, vexp):
+        check(CUMACH.word2vecNegSlice(self.opts.dim, wordsa.shape[0] // nwa, nwa, nwb, wordsa,
+                                      wordsb, modelmats, lrate, vexp, *self._slice_args(),
+                                      self.opts.doHead), "word2vecNegSlice")
+
+    def evalPositivesSlice(self, nskip, words, lb, ub, modelmats):
+        self._ret64[0:1].zero_()
+        check(CUMACH.word2vecEvalPosSlice(self.opts.dim, words.shape[0], nskip, words, lb, ub,
+                                          modelmats, *self._slice_args(), self._ret64[0:1]),
+              "word2vecEvalPosSlice")
+        return float(self._ret64[0].item())
+
+    def evalNegativesSlice(self, nwa, nwb, wordsa, wordsb, modelmats):
+        self._ret64[1:2].zero_()
+        check(CUMACH.word2vecEvalNegSlice(self.opts.dim, wordsa.shape[0] // nwa, nwa, nwb, wordsa,
+                                          wordsb, modelmats, *self._slice_args(),
+                                          self._ret64[1:2]), "word2vecEvalNegSlice")
+        return float(self._ret64[1].item())
+
     # ---- Word2Vec.dobatch / evalbatch ---------------------------------------------------
     def dobatch(self, mats, ipass, pos):
         o = self.opts
@@ -194,6 +253,12 @@ class Word2Vec:
         words, lb, ub, trandwords, goodwords = self._index_arrays(mats)
         lrpos = lrate
         lrneg = lrpos if o.eqPosNeg else lrpos / o.nneg
+        if self._sliced():
+            self.procPositivesSlice(o.nskip, words, lb, ub, self.modelmats, lrpos, o.vexp)
+            if goodwords.shape[0] > 0:
+                self.procNegativesSlice(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats,
+                                        lrneg, o.vexp)
+            return
         self.procPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0], lrpos,
                            o.vexp)
         if goodwords.shape[0] > 0:
@@ -207,9 +272,13 @@ class Word2Vec:
         words, lb, ub, trandwords, goodwords = self._index_arrays(mats)
         if goodwords.shape[0] == 0:
             return 0.0
-        epos = self.evalPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0])
-        eneg = self.evalNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
-                                  self.modelmats[0])
+        if self._sliced():
+            epos = self.evalPositivesSlice(o.nskip, words, lb, ub, self.modelmats)
+            eneg = self.evalNegativesSlice(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats)
+        else:
+            epos = self.evalPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0])
+            eneg = self.evalNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
+                                      self.modelmats[0])
         return (epos + eneg / (1 if o.eqPosNeg else o.nneg)) / goodwords.shape[0]
 
     # ---- Learner.nextPass, reduced to what Word2Vec uses (no updater, no mixins) ---------

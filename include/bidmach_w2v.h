@@ -53,6 +53,38 @@ int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float 
 int word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, int *WA, int *WB, float *A,
                     float *B, float lrate, float vexp);
 
+/* Sliced, multi-part models.  Device counterparts of the reference's CPU-only
+ * CPUMACH.word2vecPosSlice / word2vecNegSlice (CPUMACH.java:14,19; BIDMach_CPUMACH.c:80-184,
+ * :267-366; dispatched from Word2Vec.scala:404-467) and of its Scala-only forward twins
+ * evalPosCPUslice / evalNegCPUslice (Word2Vec.scala:1007-1069, :1134-1200).  Same argument lists
+ * with the thread count dropped and the length of MM added (a C array has none).
+ *
+ * MM is a HOST array of nmats DEVICE pointers, the reference's modelmats: part m of the packed
+ * model has its B table (nrows x maxCols, column-major) at MM[2m] and its A table at MM[2m+1];
+ * with dualMode != 0 the parts start at MM[2] and MM[0], MM[1] are not touched.  At most
+ * w2v_max_slice_parts() parts.  Word id w lives in packed column w if w < nHead, else
+ * nHead + (w - nHead) / nslices, and is resident iff w < nHead or w % nslices == islice
+ * (mapIndx, BIDMach_CPUMACH.c:80-88).  A pair is trained iff both words are resident and one of
+ * them is a tail word of this slice, or both are head words and doHead > 1; a column is written
+ * iff it is a tail word of this slice, or a head word and doHead > 0.  The forward twins score
+ * the pairs whose two words are resident and ADD the sum into the device double Retval[0].
+ * Deviation: inside a part the column is packed - (packed / maxCols) * maxCols for either value of
+ * dualMode (the reference's expression, :87, points maxCols columns before the part when
+ * dualMode is set). */
+int word2vecPosSlice(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float **MM,
+                     int nmats, float lrate, float vexp, int islice, int nslices, int maxCols,
+                     int nHead, int dualMode, int doHead);
+int word2vecNegSlice(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float **MM,
+                     int nmats, float lrate, float vexp, int islice, int nslices, int maxCols,
+                     int nHead, int dualMode, int doHead);
+int word2vecEvalPosSlice(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float **MM,
+                         int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+                         double *Retval);
+int word2vecEvalNegSlice(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float **MM,
+                         int nmats, int islice, int nslices, int maxCols, int nHead, int dualMode,
+                         double *Retval);
+int w2v_max_slice_parts(void);
+
 /* Replaces word2vecEvalPos, MatKernel.hpp:83 / DNN127.cu:1485-1516; arithmetic of
  * BIDMach_CPUMACH.c:368-427.  Adds sum(log(max(sigmoid(a.b), floor))) over the valid pairs into
  * the device float Retval[0] (the caller clears it first, Word2Vec.scala:476). */

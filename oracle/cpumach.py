@@ -2,7 +2,7 @@
 
 TEST INFRASTRUCTURE: only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg
 import this module.  The method names and argument lists are those of
-src/main/java/edu/berkeley/bid/CPUMACH.java:12,17,26,28 of the reference (numpy arrays stand
+src/main/java/edu/berkeley/bid/CPUMACH.java:12,14,17,19,26,28 of the reference (numpy arrays stand
 in for Java primitive arrays; A and B are updated in place).
 """
 import ctypes
@@ -47,6 +47,19 @@ def _load():
     lib.oracle_word2vecEvalPos.restype = cd
     lib.oracle_word2vecEvalNeg.argtypes = [ci, ci, ci, ci, ip, ip, fp, fp, cd, ci]
     lib.oracle_word2vecEvalNeg.restype = cd
+    fpp = ctypes.POINTER(fp)
+    lib.oracle_word2vecPosSlice.argtypes = [ci, ci, ci, ip, ip, ip, fpp, cf, cf, ci,
+                                            ci, ci, ci, ci, ci, ci]
+    lib.oracle_word2vecPosSlice.restype = None
+    lib.oracle_word2vecNegSlice.argtypes = [ci, ci, ci, ci, ip, ip, fpp, cf, cf, ci,
+                                            ci, ci, ci, ci, ci, ci]
+    lib.oracle_word2vecNegSlice.restype = None
+    lib.oracle_word2vecEvalPosSlice.argtypes = [ci, ci, ci, ip, ip, ip, fpp, cd, ci,
+                                                ci, ci, ci, ci, ci]
+    lib.oracle_word2vecEvalPosSlice.restype = cd
+    lib.oracle_word2vecEvalNegSlice.argtypes = [ci, ci, ci, ci, ip, ip, fpp, cd, ci,
+                                                ci, ci, ci, ci, ci]
+    lib.oracle_word2vecEvalNegSlice.restype = cd
     lib.oracle_max_threads.restype = ci
     _lib = lib
     return lib
@@ -60,6 +73,14 @@ def _i(a):
 def _f(a):
     assert a.dtype == np.float32 and (a.flags.c_contiguous or a.flags.f_contiguous)
     return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def _mm(mats):
+    """float** over a list of model matrices (B of part m at 2m, A at 2m+1)."""
+    arr = (ctypes.POINTER(ctypes.c_float) * len(mats))()
+    for k, m in enumerate(mats):
+        arr[k] = _f(m) if m is not None else None
+    return arr
 
 
 def max_threads():
@@ -98,3 +119,32 @@ class CPUMACH:
     def word2vecEvalNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, nthreads, floor=C_FLOOR):
         return float(_load().oracle_word2vecEvalNeg(nrows, ncols, nwa, nwb, _i(WA), _i(WB),
                                                     _f(A), _f(B), floor, nthreads))
+
+    # ---- sliced, multi-part models (CPUMACH.java:14,19; Scala-only forward twins) ----------
+    @staticmethod
+    def word2vecPosSlice(nrows, ncols, skip, W, LB, UB, MM, lrate, vexp, nthreads, islice,
+                         nslices, maxCols, nHead, dualMode, doHead):
+        _load().oracle_word2vecPosSlice(nrows, ncols, skip, _i(W), _i(LB), _i(UB), _mm(MM), lrate,
+                                        vexp, nthreads, islice, nslices, maxCols, nHead,
+                                        int(dualMode), doHead)
+
+    @staticmethod
+    def word2vecNegSlice(nrows, ncols, nwa, nwb, WA, WB, MM, lrate, vexp, nthreads, islice,
+                         nslices, maxCols, nHead, dualMode, doHead):
+        _load().oracle_word2vecNegSlice(nrows, ncols, nwa, nwb, _i(WA), _i(WB), _mm(MM), lrate,
+                                        vexp, nthreads, islice, nslices, maxCols, nHead,
+                                        int(dualMode), doHead)
+
+    @staticmethod
+    def word2vecEvalPosSlice(nrows, ncols, skip, W, LB, UB, MM, nthreads, islice, nslices,
+                             maxCols, nHead, dualMode, floor=SCALA_FLOOR):
+        return float(_load().oracle_word2vecEvalPosSlice(
+            nrows, ncols, skip, _i(W), _i(LB), _i(UB), _mm(MM), floor, nthreads, islice, nslices,
+            maxCols, nHead, int(dualMode)))
+
+    @staticmethod
+    def word2vecEvalNegSlice(nrows, ncols, nwa, nwb, WA, WB, MM, nthreads, islice, nslices,
+                             maxCols, nHead, dualMode, floor=SCALA_FLOOR):
+        return float(_load().oracle_word2vecEvalNegSlice(
+            nrows, ncols, nwa, nwb, _i(WA), _i(WB), _mm(MM), floor, nthreads, islice, nslices,
+            maxCols, nHead, int(dualMode)))

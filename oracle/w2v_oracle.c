@@ -13,6 +13,9 @@
  *   oracle_word2vecNegFilt  <- the same arithmetic as word2vecNeg under the id filter of the
  *                              reference's GPU-only __word2vecNegFilt (jni/src/DNN127.cu:690-711):
  *                              a word id >= nwords drops every pair it takes part in
+ *   oracle_word2vec{Pos,Neg}Slice     <- :80-184, :267-366 (multi-part, sliced model)
+ *   oracle_word2vecEval{Pos,Neg}Slice <- the Scala-only forward twins,
+ *                              src/main/scala/BIDMach/networks/Word2Vec.scala:1007-1069, :1134-1200
  * with the JNI array pinning replaced by plain pointers.  Arithmetic order is
  * kept (fp32 multiply then add in ascending row order, exp/pow/log in double,
  * B updated inside the window loop, A after it) so that a single-threaded run
@@ -24,6 +27,9 @@
  *     wherever the reference's product does not overflow;
  *   - the Eval accumulators start at zero; the reference leaves `double sum`
  *     uninitialised (:379, :439);
+ *   - in the sliced variants the column inside a part is newi - (newi / maxCols) * maxCols; the
+ *     reference subtracts (newi / maxCols + offset) * maxCols (:87), which with dualMode (offset 1)
+ *     points maxCols columns before the start of the part;
  *   - the Eval floor is a parameter (the C reference uses 1e-40, the Scala and
  *     CUDA twins 1e-20: Word2Vec.scala:995,1123, DNN127.cu:310,916).
  *
@@ -226,6 +232,241 @@ double oracle_word2vecEvalNeg(int nrows, int ncols, int nwa, int nwb, const int 
           for (c = 0; c < nrows; c++) cv += A[c + ia] * B[c + ib];
           cv = oracle_sigmoid(cv);
           dv += log(fmax(1.0 - (double)cv, floorv));
+        }
+      }
+    }
+    pv[ithread] = dv;
+  }
+  for (i = 0; i < nthreads; i++) sum += pv[i];
+  free(pv);
+  return sum;
+}
+
+/* Where word `indx` of a sliced, multi-part model lives (BIDMach_CPUMACH.c:80-88): ids below nhead
+ * ("head") keep their column and exist on every slice; the others ("tail") are dealt round-robin
+ * to nslices slices and packed after the head.  Part m of the model holds columns
+ * [m*maxcols, (m+1)*maxcols); its B table is MM[2*(m+offset)], its A table MM[2*(m+offset)+1]. */
+static void oracle_map_index(int *mm, int64_t *ii, int *ismine, int *ishead, int indx, int islice,
+                             int nslices, int nhead, int maxcols, int nrows, int offset) {
+  int newi = indx;
+  int part;
+  if (indx >= nhead) newi = (indx - nhead) / nslices + nhead;
+  part = newi / maxcols;
+  *mm = part + offset;
+  *ismine = (indx >= nhead) && (indx % nslices == islice);
+  *ishead = (indx < nhead);
+  *ii = (int64_t)nrows * (newi - part * maxcols);
+}
+
+static int oracle_pair_trained(int aismine, int aishead, int bismine, int bishead, int doHead) {
+  /* BIDMach_CPUMACH.c:137, :315 */
+  return (doHead > 1 && aishead && bishead) || (aismine && bishead) || (bismine && aishead) ||
+         (aismine && bismine);
+}
+
+void oracle_word2vecPosSlice(int nrows, int ncols, int skip, const int *W, const int *LB,
+                             const int *UB, float **MM, float lrate, float vexp, int nthreads,
+                             int islice, int nslices, int maxCols, int nHead, int dualMode,
+                             int doHead) {
+  int ithread;
+  const int offset = dualMode ? 1 : 0;
+  (void)skip;
+#pragma omp parallel for num_threads(nthreads)
+  for (ithread = 0; ithread < nthreads; ithread++) {
+    int istart = (int)((1L * ithread * ncols) / nthreads);
+    int iend = (int)((1L * (ithread + 1) * ncols) / nthreads);
+    int i, j, c, iac, ibc, touched;
+    int64_t ia, ib;
+    int aismine, bismine, aishead, bishead, ma, mb;
+    float cv, ascale, bscale;
+    float *A, *B;
+    float *daa = (float *)malloc((size_t)nrows * sizeof(float));
+
+    for (i = istart; i < iend; i++) {
+      iac = W[i];
+      if (iac >= 0) {
+        oracle_map_index(&ma, &ia, &aismine, &aishead, iac, islice, nslices, nHead, maxCols, nrows,
+                         offset);
+        A = MM[2 * ma + 1];
+        ascale = pow(1 + iac, vexp);
+        for (c = 0; c < nrows; c++) daa[c] = 0;
+        touched = 0;
+        for (j = LB[i]; j <= UB[i]; j++) {
+          if (j != 0 && i + j >= 0 && i + j < ncols) {
+            ibc = W[i + j];
+            if (ibc >= 0) {
+              oracle_map_index(&mb, &ib, &bismine, &bishead, ibc, islice, nslices, nHead, maxCols,
+                               nrows, offset);
+              B = MM[2 * mb];
+              bscale = pow(1 + ibc, vexp);
+              if (oracle_pair_trained(aismine, aishead, bismine, bishead, doHead)) {
+                touched = 1;
+                cv = 0;
+                for (c = 0; c < nrows; c++) cv += A[c + ia] * B[c + ib];
+                cv = oracle_sigmoid(cv);
+                cv = lrate * (1.0f - cv);
+                for (c = 0; c < nrows; c++) daa[c] += ascale * cv * B[c + ib];
+                if (bismine || (bishead && doHead)) {
+                  for (c = 0; c < nrows; c++) B[c + ib] += bscale * cv * A[c + ia];
+                }
+              }
+            }
+          }
+        }
+        if (touched && (aismine || (aishead && doHead))) {
+          for (c = 0; c < nrows; c++) A[c + ia] += daa[c];
+        }
+      }
+    }
+    free(daa);
+  }
+}
+
+void oracle_word2vecNegSlice(int nrows, int ncols, int nwa, int nwb, const int *WA, const int *WB,
+                             float **MM, float lrate, float vexp, int nthreads, int islice,
+                             int nslices, int maxCols, int nHead, int dualMode, int doHead) {
+  int ithread;
+  const int offset = dualMode ? 1 : 0;
+#pragma omp parallel for num_threads(nthreads)
+  for (ithread = 0; ithread < nthreads; ithread++) {
+    int i, j, k, c, iac, ibc;
+    int64_t ia, ib, ja;
+    float cv, ascale, bscale;
+    float *A, *B;
+    int aismine, bismine, aishead, bishead, ma, mb;
+    int istart = (int)((1L * ithread * ncols) / nthreads);
+    int iend = (int)((1L * (ithread + 1) * ncols) / nthreads);
+    float *daa = (float *)malloc((size_t)nwa * nrows * sizeof(float));
+    float *dbb = (float *)malloc((size_t)nrows * sizeof(float));
+
+    for (i = istart; i < iend; i++) {
+      for (c = 0; c < nwa * nrows; c++) daa[c] = 0;
+      for (k = 0; k < nwb; k++) {
+        ibc = WB[k + (int64_t)i * nwb];
+        oracle_map_index(&mb, &ib, &bismine, &bishead, ibc, islice, nslices, nHead, maxCols, nrows,
+                         offset);
+        B = MM[2 * mb];
+        bscale = pow(1 + ibc, vexp);
+        for (c = 0; c < nrows; c++) dbb[c] = 0;
+        for (j = 0; j < nwa; j++) {
+          iac = WA[j + (int64_t)i * nwa];
+          oracle_map_index(&ma, &ia, &aismine, &aishead, iac, islice, nslices, nHead, maxCols, nrows,
+                           offset);
+          A = MM[2 * ma + 1];
+          ascale = pow(1 + iac, vexp);
+          if (oracle_pair_trained(aismine, aishead, bismine, bishead, doHead)) {
+            cv = 0;
+            for (c = 0; c < nrows; c++) cv += A[c + ia] * B[c + ib];
+            cv = oracle_sigmoid(cv);
+            cv = -lrate * cv;
+            ja = (int64_t)j * nrows;
+            for (c = 0; c < nrows; c++) {
+              dbb[c] += bscale * cv * A[c + ia];
+              daa[c + ja] += ascale * cv * B[c + ib];
+            }
+          }
+        }
+        if (bismine || (bishead && doHead)) {
+          for (c = 0; c < nrows; c++) B[c + ib] += dbb[c];
+        }
+      }
+      for (j = 0; j < nwa; j++) {
+        ja = (int64_t)j * nrows;
+        iac = WA[j + (int64_t)i * nwa];
+        oracle_map_index(&ma, &ia, &aismine, &aishead, iac, islice, nslices, nHead, maxCols, nrows,
+                         offset);
+        A = MM[2 * ma + 1];
+        if (aismine || (aishead && doHead)) {
+          for (c = 0; c < nrows; c++) A[c + ia] += daa[c + ja];
+        }
+      }
+    }
+    free(dbb);
+    free(daa);
+  }
+}
+
+/* Word2Vec.scala:1007-1069: a pair is scored iff both words are resident (mine or head). */
+double oracle_word2vecEvalPosSlice(int nrows, int ncols, int skip, const int *W, const int *LB,
+                                   const int *UB, float **MM, double floorv, int nthreads,
+                                   int islice, int nslices, int maxCols, int nHead, int dualMode) {
+  int i, ithread;
+  const int offset = dualMode ? 1 : 0;
+  double *pv = (double *)malloc((size_t)nthreads * sizeof(double));
+  double sum = 0;
+  (void)skip;
+#pragma omp parallel for num_threads(nthreads)
+  for (ithread = 0; ithread < nthreads; ithread++) {
+    int istart = (int)((1L * ithread * ncols) / nthreads);
+    int iend = (int)((1L * (ithread + 1) * ncols) / nthreads);
+    int ii, j, c, ma, mb, aismine, aishead, bismine, bishead;
+    int64_t ia, ib;
+    float cv;
+    const float *A, *B;
+    double dv = 0;
+    for (ii = istart; ii < iend; ii++) {
+      if (W[ii] >= 0) {
+        oracle_map_index(&ma, &ia, &aismine, &aishead, W[ii], islice, nslices, nHead, maxCols,
+                         nrows, offset);
+        if (aismine || aishead) {
+          A = MM[2 * ma + 1];
+          for (j = LB[ii]; j <= UB[ii]; j++) {
+            if (j != 0 && ii + j >= 0 && ii + j < ncols && W[ii + j] >= 0) {
+              oracle_map_index(&mb, &ib, &bismine, &bishead, W[ii + j], islice, nslices, nHead,
+                               maxCols, nrows, offset);
+              if (bismine || bishead) {
+                B = MM[2 * mb];
+                cv = 0;
+                for (c = 0; c < nrows; c++) cv += A[c + ia] * B[c + ib];
+                cv = oracle_sigmoid(cv);
+                dv += log(fmax((double)cv, floorv));
+              }
+            }
+          }
+        }
+      }
+    }
+    pv[ithread] = dv;
+  }
+  for (i = 0; i < nthreads; i++) sum += pv[i];
+  free(pv);
+  return sum;
+}
+
+/* Word2Vec.scala:1134-1200 */
+double oracle_word2vecEvalNegSlice(int nrows, int ncols, int nwa, int nwb, const int *WA,
+                                   const int *WB, float **MM, double floorv, int nthreads,
+                                   int islice, int nslices, int maxCols, int nHead, int dualMode) {
+  int i, ithread;
+  const int offset = dualMode ? 1 : 0;
+  double *pv = (double *)malloc((size_t)nthreads * sizeof(double));
+  double sum = 0;
+#pragma omp parallel for num_threads(nthreads)
+  for (ithread = 0; ithread < nthreads; ithread++) {
+    int ii, j, k, c, ma, mb, aismine, aishead, bismine, bishead;
+    int64_t ia, ib;
+    float cv;
+    const float *A, *B;
+    double dv = 0;
+    int istart = (int)((1L * ithread * ncols) / nthreads);
+    int iend = (int)((1L * (ithread + 1) * ncols) / nthreads);
+    for (ii = istart; ii < iend; ii++) {
+      for (k = 0; k < nwb; k++) {
+        oracle_map_index(&mb, &ib, &bismine, &bishead, WB[k + (int64_t)ii * nwb], islice, nslices,
+                         nHead, maxCols, nrows, offset);
+        if (bismine || bishead) {
+          B = MM[2 * mb];
+          for (j = 0; j < nwa; j++) {
+            oracle_map_index(&ma, &ia, &aismine, &aishead, WA[j + (int64_t)ii * nwa], islice,
+                             nslices, nHead, maxCols, nrows, offset);
+            if (aismine || aishead) {
+              A = MM[2 * ma + 1];
+              cv = 0;
+              for (c = 0; c < nrows; c++) cv += A[c + ia] * B[c + ib];
+              cv = oracle_sigmoid(cv);
+              dv += log(fmax(1.0 - (double)cv, floorv));
+            }
+          }
         }
       }
     }

@@ -104,3 +104,50 @@ def test_odd_sized_minibatch_is_skipped():
     m.dobatch(mats, 0, 1000)
     assert torch.equal(before[0], m.modelmats[0]) and torch.equal(before[1], m.modelmats[1])
     assert m.evalbatch(mats, 0, 1000) == 0.0
+
+
+@pytest.mark.parametrize("dual", [False, True])
+def test_sliced_multipart_model_matches_oracle_step(oracle, dual):
+    """A two-worker, several-part model (every part its own device allocation): dobatch and
+    evalbatch go through the device Slice operators; the same step is replayed with the oracle's
+    Slice functions on the index arrays read back from the device."""
+    o = Options(vocabSize=4000, dim=64, batchSize=6000, lrate=0.005, vexp=0.5, seed=4,
+                nSlices=2, iSlice=1, nHeadTerms=300, maxArraySize=64 * 700, doHead=1,
+                dualMode=dual)
+    m = Word2Vec(o)
+    m.init()
+    assert m.maxCols == 700 and m.nmmats == 4        # 300 + 1 + 3699 // 2 = 2150 columns
+    assert len(m.modelmats) == 2 * (4 + (1 if dual else 0))
+    assert [x.shape[0] for x in m.modelmats[-8::2]] == [700, 700, 700, 50]
+    host = [x.cpu().numpy().copy() for x in m.modelmats]
+    mats = make_stream(6000, 4000, seed=22)
+    m.dobatch(mats, 0, 6000)
+    b = m._wm
+    npairs, G = b["counts"].cpu().tolist()
+    words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
+    negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
+    ctx = b["ctx"].cpu().numpy()[:G * o.nreuse].copy()
+    sl = (1, 1, 2, 700, 300, dual)
+    oracle.word2vecPosSlice(64, 6000, o.nskip, words, lb, ub, host, 0.005, 0.5, *sl, 1)
+    oracle.word2vecNegSlice(64, G, o.nneg, o.nreuse, negs, ctx, host, 0.005 / o.nneg, 0.5, *sl, 1)
+    moved = 0.0
+    for g, h in zip(m.modelmats, host):
+        assert np.abs(g.cpu().numpy() - h).max() < 2e-3
+        moved = max(moved, float(np.abs(h).max()))
+    if dual:      # the leading pair is not part of the sliced model
+        assert np.array_equal(m.modelmats[1].cpu().numpy(), np.zeros_like(host[1]))
+    held = make_stream(6000, 4000, seed=23)
+    got = m.evalbatch(held, 0, 12000)
+    b = m._wm
+    npairs, G = b["counts"].cpu().tolist()
+    words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
+    negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
+    ctx = b["ctx"].cpu().numpy()[:G * o.nreuse].copy()
+    host = [x.cpu().numpy().copy() for x in m.modelmats]
+    epos = oracle.word2vecEvalPosSlice(64, 6000, o.nskip, words, lb, ub, host, 4, 1, 2, 700, 300,
+                                       dual, floor=1e-40)
+    eneg = oracle.word2vecEvalNegSlice(64, G, o.nneg, o.nreuse, negs, ctx, host, 4, 1, 2, 700, 300,
+                                       dual, floor=1e-40)
+    want = (epos + eneg / o.nneg) / ctx.shape[0]
+    assert want < -0.05
+    assert got == pytest.approx(want, rel=1e-5)

@@ -112,3 +112,24 @@ def test_iflip_swaps_rows():
     b = model(vocabSize=V, wsample=1.0, seed=4, iflip=True).wordMats(mats[::-1])
     for x, y in zip(a, b):
         assert np.array_equal(x, y)
+
+
+def test_sliced_model_list_has_the_reference_shape():
+    """Word2Vec.scala:100-131: columns on this worker, number of parts, dual-mode list."""
+    from bidmach_amd.word2vec import Options, Word2Vec
+    o = Options(vocabSize=1000, dim=8, nSlices=3, iSlice=2, nHeadTerms=100, maxArraySize=8 * 150)
+    m = Word2Vec(o, device="cpu")
+    m.init()
+    actual = 100 + 1 + (1000 - 100 - 1) // 3
+    assert actual == 400 and m.maxCols == 150 and m.nmmats == 3 and m._sliced()
+    assert [tuple(x.shape) for x in m.modelmats] == [(150, 8)] * 4 + [(100, 8)] * 2
+    assert all(float(x.abs().max()) == 0.0 for x in m.modelmats[1::2])       # A tables start at 0
+    assert all(0 < float(x.abs().max()) <= 0.5 / 8 for x in m.modelmats[0::2])
+    o.dualMode = True
+    m = Word2Vec(o, device="cpu")
+    m.init()
+    assert len(m.modelmats) == 8 and m._dual
+    assert (m.modelmats[0] == m.modelmats[2]).all() and (m.modelmats[1] == m.modelmats[3]).all()
+    plain = Word2Vec(Options(vocabSize=1000, dim=8), device="cpu")
+    plain.init()
+    assert not plain._sliced() and [tuple(x.shape) for x in plain.modelmats] == [(1000, 8)] * 2
