@@ -108,6 +108,9 @@ def main():
     ap.add_argument("--mode", default="train", choices=["train", "eval"],
                     help="train: word2vecPos + word2vecNeg (the headline); eval: forward-only "
                          "word2vecEvalPos + word2vecEvalNeg")
+    ap.add_argument("--parts", type=int, default=0,
+                    help="train mode only: cut each table into this many separate allocations and "
+                         "run the step through word2vecPosSlice + word2vecNegSlice (one worker)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run one plain 1 GiB device copy before the timed region (gives a "
@@ -152,6 +155,12 @@ def main():
         A.normal_(0.0, 0.1)
         B.normal_(0.0, 0.1)
     ret = torch.zeros(2, dtype=torch.float32, device="cuda")
+    MM, maxcols = None, 0
+    if args.parts > 0 and not evaluating:
+        maxcols = (V + args.parts - 1) // args.parts
+        MM = []
+        for c0 in range(0, V, maxcols):
+            MM += [B[c0:c0 + maxcols].clone(), A[c0:c0 + maxcols].clone()]
 
     def step(s, timers=None):
         mb, hmb = dev_mbs[s % ndistinct], host_mbs[s % ndistinct]
@@ -161,6 +170,10 @@ def main():
         if evaluating:
             check(CUMACH.word2vecEvalPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B,
                                               ret[0:1]), "word2vecEvalPos")
+        elif MM:
+            check(CUMACH.word2vecPosSlice(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], MM, lr,
+                                          args.vexp, 0, 1, maxcols, 0, False, 1),
+                  "word2vecPosSlice")
         else:
             check(CUMACH.word2vecPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr,
                                           args.vexp), "word2vecPos")
@@ -170,6 +183,10 @@ def main():
         if evaluating:
             check(CUMACH.word2vecEvalNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                               mb["WB"], A, B, ret[1:2]), "word2vecEvalNeg")
+        elif MM:
+            check(CUMACH.word2vecNegSlice(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
+                                          mb["WB"], MM, lr / cfg["nneg"], args.vexp, 0, 1, maxcols,
+                                          0, False, 1), "word2vecNegSlice")
         else:
             check(CUMACH.word2vecNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                           mb["WB"], A, B, lr / cfg["nneg"], args.vexp),
@@ -209,6 +226,8 @@ def main():
     step_gbps = (avg_pos_b + avg_neg_b) / ((avg_pos_ms + avg_neg_ms) * 1e-3) / 1e9
 
     assert bool(torch.isfinite(A).all()) and bool(torch.isfinite(B).all()), "tables diverged"
+    if MM:
+        assert all(bool(torch.isfinite(m).all()) for m in MM), "tables diverged"
 
     words_per_s = K * n / elapsed
     out = {
@@ -252,6 +271,10 @@ def main():
 
     if evaluating:
         out["config"]["mode"] = "eval"
+        out["roofline"]["traffic"] = None
+    if MM:
+        out["config"]["parts"] = len(MM) // 2
+        out["config"]["operators"] = "word2vecPosSlice+word2vecNegSlice"
         out["roofline"]["traffic"] = None
     if not args.no_cpu_baseline and not evaluating:
         threads = host_threads()

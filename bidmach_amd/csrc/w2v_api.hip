@@ -171,7 +171,7 @@ bool slice_map(float** MM, int nmats, int islice, int nslices, int maxCols, int 
   return true;
 }
 
-int pos_slice_impl(int nrows, int ncols, int* W, int* LB, int* UB, float** MM, int nmats,
+int pos_slice_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float** MM, int nmats,
                    float lrate, float vexp, int islice, int nslices, int maxCols, int nHead,
                    int dualMode, int doHead) {
   w2v::SliceMap m;
@@ -180,7 +180,11 @@ int pos_slice_impl(int nrows, int ncols, int* W, int* LB, int* UB, float** MM, i
     return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_slice_pos(t_state.stream, nrows, ncols, W, LB, UB, m, lrate, vexp),
+  w2v::Shadow shadow{};
+  hipError_t err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_slice_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, m, lrate,
+                                      vexp, shadow),
                 true);
 }
 
@@ -193,8 +197,11 @@ int neg_slice_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, flo
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB) return (int)hipErrorInvalidValue;
+  w2v::Shadow shadow{};
+  hipError_t err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_slice_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate,
-                                      vexp),
+                                      vexp, shadow),
                 true);
 }
 
@@ -259,9 +266,8 @@ int word2vecNegFilt(int nrows, int ncols, int nwords, int nwa, int nwb, int* WA,
 int word2vecPosSlice(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float** MM,
                      int nmats, float lrate, float vexp, int islice, int nslices, int maxCols,
                      int nHead, int dualMode, int doHead) {
-  (void)shift;
-  return pos_slice_impl(nrows, ncols, W, LB, UB, MM, nmats, lrate, vexp, islice, nslices, maxCols,
-                        nHead, dualMode, doHead);
+  return pos_slice_impl(nrows, ncols, shift, W, LB, UB, MM, nmats, lrate, vexp, islice, nslices,
+                        maxCols, nHead, dualMode, doHead);
 }
 
 int word2vecNegSlice(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float** MM,

@@ -201,6 +201,106 @@ __device__ __forceinline__ float* scatter_target(float* table, float* shadow, in
   return shadow + ((int64_t)slot * kHotWords + w) * d;
 }
 
+// ---- where a word's column lives -------------------------------------------------------------
+//
+// The kernels that serve both the single-table model and the sliced, multi-part model see the
+// model through a small policy object: it turns a word id into a ColRef and answers the two
+// questions the sliced model adds (is this pair trained? may this column be written?).
+
+constexpr int kMine = 1;  // sliced model: a tail word this worker owns; single table: any word
+constexpr int kHead = 2;  // sliced model: a head word, resident on every worker
+
+struct ColRef {
+  float* col;  // start of the column
+  int hot;     // index of its shadow copies, or -1 if the column has none
+  int flags;   // 0: not resident (skip the word), else kMine or kHead
+};
+
+template <int R>
+__device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const float* shadow,
+                                             int lane, int d) {
+  load_col<R>(x, ref.col, lane, d);
+  if (ref.hot >= 0) {
+    const int copies = shadow_copies(ref.hot);
+#pragma unroll 1
+    for (int s = 0; s < copies; s += 2) {
+      float y0[R], y1[R];
+      load_col<R>(y0, shadow + ((int64_t)s * kHotWords + ref.hot) * d, lane, d);
+      load_col<R>(y1, shadow + ((int64_t)(s + 1) * kHotWords + ref.hot) * d, lane, d);
+#pragma unroll
+      for (int r = 0; r < R; ++r) x[r] += y0[r] + y1[r];
+    }
+  }
+}
+
+// Column that receives the atomics for `ref` from workgroup number `wg`.
+__device__ __forceinline__ float* scatter_ref(const ColRef& ref, float* shadow, int wg, int d) {
+  if (ref.hot < 0) return ref.col;
+  const int slot = wg & (shadow_copies(ref.hot) - 1);
+  return shadow + ((int64_t)slot * kHotWords + ref.hot) * d;
+}
+
+// One pair of tables: word w is column w of A / of B; every pair is trained, every column written.
+struct PlainTables {
+  float* A;
+  float* B;
+  static constexpr bool kSliced = false;
+  __device__ __forceinline__ ColRef a(int w, int d) const {
+    return ColRef{A + (int64_t)w * d, w < kHotWords ? w : -1, w >= 0 ? kMine : 0};
+  }
+  __device__ __forceinline__ ColRef b(int w, int d) const {
+    return ColRef{B + (int64_t)w * d, w < kHotWords ? w : -1, w >= 0 ? kMine : 0};
+  }
+  __device__ __forceinline__ bool trained(int, int) const { return true; }
+  __device__ __forceinline__ bool written(int) const { return true; }
+};
+
+// A sliced, multi-part model (jni/src/BIDMach_CPUMACH.c:80-88 of the reference).  The vocabulary
+// is split over nslices workers: ids below nhead ("head") are resident on every worker, an id
+// >= nhead ("tail") on worker id % nslices only.  A worker packs its resident words densely
+// (head, then its tail words in id order: packed column nhead + (id - nhead) / nslices) and cuts
+// the packed table into parts of maxcols columns, each part a separate allocation; part m has
+// its B table at mats[2m] and its A table at mats[2m+1].  Passed to kernels by value.
+constexpr int kMaxSliceParts = 32;
+struct SliceMap {
+  float* mats[2 * kMaxSliceParts];
+  int nparts;   // parts present; a word whose packed column falls beyond them is skipped
+  int islice;   // this worker
+  int nslices;  // workers the tail of the vocabulary is dealt to
+  int nhead;    // ids below this are resident on every worker
+  int maxcols;  // columns per part
+  int dohead;   // 0: head columns read-only, 1: written, 2: written and head-head pairs trained
+};
+
+struct SlicedTables {
+  SliceMap m;
+  static constexpr bool kSliced = true;
+  // which: 0 = B table of the part, 1 = A table
+  __device__ __forceinline__ ColRef place(int w, int which, int d) const {
+    ColRef r{nullptr, -1, 0};
+    if (w < 0) return r;
+    const bool head = w < m.nhead;
+    const bool mine = !head && (w % m.nslices == m.islice);
+    if (!head && !mine) return r;
+    const int packed = head ? w : (w - m.nhead) / m.nslices + m.nhead;
+    const int part = packed / m.maxcols;
+    if (part >= m.nparts) return r;
+    r.col = m.mats[2 * part + which] + (int64_t)(packed - part * m.maxcols) * d;
+    r.hot = (part == 0 && packed < kHotWords) ? packed : -1;  // the first columns of part 0
+    r.flags = head ? kHead : kMine;
+    return r;
+  }
+  __device__ __forceinline__ ColRef a(int w, int d) const { return place(w, 1, d); }
+  __device__ __forceinline__ ColRef b(int w, int d) const { return place(w, 0, d); }
+  // Rules of the reference (:137-157, :315-349); both words are resident when these are asked.
+  __device__ __forceinline__ bool trained(int fa, int fb) const {
+    return (((fa | fb) & kMine) != 0) || m.dohead > 1;
+  }
+  __device__ __forceinline__ bool written(int f) const {
+    return f == kMine || (f == kHead && m.dohead > 0);
+  }
+};
+
 // Block-level sum of one double per wave, written as one partial per block.
 __device__ __forceinline__ void block_store_partial(double wave_total, double* __restrict__ partials) {
   __shared__ double s_part[kWavesPerBlock];

@@ -64,28 +64,23 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
 hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, float* Retval32,
                            double* Retval64);
 
-// A sliced, multi-part model as the kernels see it: part m has its B table at mats[2m] and its A
-// table at mats[2m+1], each of maxcols columns (the last part may be shorter).  Passed by value.
-constexpr int kMaxSliceParts = 32;
-struct SliceMap {
-  float* mats[2 * kMaxSliceParts];
-  int nparts;   // parts present; a word whose packed column falls beyond them is skipped
-  int islice;   // this worker
-  int nslices;  // workers the tail of the vocabulary is dealt to
-  int nhead;    // ids below this are resident on every worker
-  int maxcols;  // columns per part
-  int dohead;   // 0: head columns read-only, 1: written, 2: written and head-head pairs trained
-};
-
 int max_slice_parts();
 // Capacity the Eval launchers below need in `partials`.
 int64_t slice_eval_partials_needed();
 
-hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                            const int* UB, const SliceMap& m, float lrate, float vexp);
+// Update passes over a sliced, multi-part model (SliceMap, w2v_device.h).  The shadow buffers
+// serve the first kHotWords packed columns of part 0 and are left zeroed.
+hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                            const int* LB, const int* UB, const SliceMap& m, float lrate,
+                            float vexp, Shadow shadow);
 hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                             const int* WA, const int* WB, const SliceMap& m, float lrate,
-                            float vexp);
+                            float vexp, Shadow shadow);
+// The tiled positive pass on a sliced model; *launched is false (and nothing was enqueued) when
+// no tile fits in LDS for this nrows / shift.
+hipError_t launch_slice_pos_tiled(hipStream_t stream, int nrows, int ncols, int shift,
+                                  const int* W, const int* LB, const int* UB, const SliceMap& m,
+                                  float lrate, float vexp, Shadow shadow, bool* launched);
 hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const int* W,
                                  const int* LB, const int* UB, const SliceMap& m, double floorv,
                                  double* partials, float* Retval32, double* Retval64);

@@ -133,20 +133,24 @@ constexpr int kTileThreads = kTileWaves * kWave;
 constexpr int kMaxHalo = 31;       // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
 constexpr int kMinTilesPerWg = 64; // a workgroup walks at least this many consecutive tiles
 
-// LDS layout of a workgroup: a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh]
-// with dp = R*64 (columns zero-padded so that LDS reads need no bounds test).
+// LDS layout of a workgroup:
+//   a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh] | ft[T + 2*Sh]
+// with dp = R*64 (columns zero-padded so that LDS reads need no bounds test).  wt holds the word
+// id of a staged position (-1 if the word is skipped), ft its residency flags.
 __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
   const size_t dp = (size_t)R * kWave;
   return ((size_t)T * dp + (size_t)(T + 2 * Sh) * dp + (size_t)T * (2 * Sh + 1) +
-          (size_t)(T + 2 * Sh)) * 4;
+          2 * (size_t)(T + 2 * Sh)) * 4;
 }
 
-template <int R>
+// `tables` is PlainTables (word2vecPos) or SlicedTables (word2vecPosSlice): it places a word's
+// column and says which pairs are trained and which columns are written.
+template <int R, class Tables>
 __global__ void __launch_bounds__(kTileThreads)
 pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg,
                 const int* __restrict__ W, const int* __restrict__ LB,
-                const int* __restrict__ UB, float* A, float* B, float lrate, float vexp,
-                int smode, Shadow shadow) {
+                const int* __restrict__ UB, Tables tables, float lrate, float vexp, int smode,
+                Shadow shadow) {
   extern __shared__ float lds[];
   constexpr int dp = R * kWave;
   const int lane = threadIdx.x & 63;
@@ -156,6 +160,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
   float* const b_t = a_t + (size_t)T * dp;
   float* const G = b_t + (size_t)(T + 2 * Sh) * dp;
   int* const wt = reinterpret_cast<int*>(G + (size_t)T * gw);
+  int* const ft = wt + (T + 2 * Sh);
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
   const int64_t tile_begin = (int64_t)blockIdx.x * tiles_per_wg;
@@ -175,18 +180,24 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const int c1 = c0 + kTileWaves;
       const int w0 = W[hlo + c0];
       const int w1 = c1 < nh ? W[hlo + c1] : -1;
+      const ColRef r0 = tables.b(w0, d);
+      const ColRef r1 = tables.b(w1, d);
       float x0[R], x1[R];
-      if (w0 >= 0) load_col_hot<R>(x0, B, shadow.b, w0, lane, d);
-      if (w1 >= 0) load_col_hot<R>(x1, B, shadow.b, w1, lane, d);
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.b, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.b, lane, d);
       if (lane == 0) {
-        wt[c0] = w0;
-        if (c1 < nh) wt[c1] = w1;
+        wt[c0] = r0.flags != 0 ? w0 : -1;
+        ft[c0] = r0.flags;
+        if (c1 < nh) {
+          wt[c1] = r1.flags != 0 ? w1 : -1;
+          ft[c1] = r1.flags;
+        }
       }
-      if (w0 >= 0) {
+      if (r0.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) b_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
       }
-      if (w1 >= 0) {
+      if (r1.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) b_t[(size_t)c1 * dp + r * kWave + lane] = x1[r];
       }
@@ -195,14 +206,16 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const int c1 = c0 + kTileWaves;
       const int w0 = W[lo + c0];
       const int w1 = c1 < nc ? W[lo + c1] : -1;
+      const ColRef r0 = tables.a(w0, d);
+      const ColRef r1 = tables.a(w1, d);
       float x0[R], x1[R];
-      if (w0 >= 0) load_col_hot<R>(x0, A, shadow.a, w0, lane, d);
-      if (w1 >= 0) load_col_hot<R>(x1, A, shadow.a, w1, lane, d);
-      if (w0 >= 0) {
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.a, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.a, lane, d);
+      if (r0.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) a_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
       }
-      if (w1 >= 0) {
+      if (r1.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) a_t[(size_t)c1 * dp + r * kWave + lane] = x1[r];
       }
@@ -215,6 +228,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const int i = lo + ci;
       const int wi = wt[i - hlo];
       if (wi < 0) continue;
+      const int fi = Tables::kSliced ? ft[i - hlo] : kMine;
       const int jlo = max(LB[i], -i);
       const int jhi = min(UB[i], ncols - 1 - i);
       float a[R];
@@ -230,6 +244,9 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
         const int j = lane - Sh;
         int wl = -1;
         if (lane < gw && j != 0 && j >= jlo && j <= jhi) wl = wt[i + j - hlo];
+        if (Tables::kSliced) {
+          if (wl >= 0 && !tables.trained(fi, ft[i + j - hlo])) wl = -1;
+        }
         const unsigned long long valid = __ballot(wl >= 0);
         if (valid != 0ull) {
           float pre = 0.0f;
@@ -267,17 +284,20 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
           continue;
         }
         const int wb = W[i + j];
-        if (wb < 0) continue;
+        const ColRef rb = tables.b(wb, d);
+        if (rb.flags == 0 || !tables.trained(fi, rb.flags)) continue;
         float b[R];
-        load_col_hot<R>(b, B, shadow.b, wb, lane, d);
+        load_col_ref<R>(b, rb, shadow.b, lane, d);
         const float s = wave_sum(dot_partial<R>(a, b));
         const float g = lrate * (1.0f - sat_sigmoid(s));
         axpy<R>(daa, ascale * g, b);
-        atomic_axpy_col<R>(scatter_target(B, shadow.b, wb, slot, d),
-                           scale_of(wb, vexp, smode) * g, a, lane, d);
+        if (tables.written(rb.flags))
+          atomic_axpy_col<R>(scatter_ref(rb, shadow.b, slot, d), scale_of(wb, vexp, smode) * g, a,
+                             lane, d);
         touched = true;
       }
-      if (touched) atomic_add_col<R>(scatter_target(A, shadow.a, wi, slot, d), daa, lane, d);
+      if (touched && tables.written(fi))
+        atomic_add_col<R>(scatter_ref(tables.a(wi, d), shadow.a, slot, d), daa, lane, d);
     }
     __syncthreads();
 
@@ -285,6 +305,9 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
     for (int c = wave; c < nh; c += kTileWaves) {
       const int wp = wt[c];
       if (wp < 0) continue;
+      if (Tables::kSliced) {
+        if (!tables.written(ft[c])) continue;
+      }
       const int p = hlo + c;
       // lane l looks at centre i = p - Sh + l; its g for this position sits at offset p - i
       const int i = p - Sh + lane;
@@ -302,8 +325,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
 #pragma unroll
         for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, acol[r * kWave], dbb[r]);
       }
-      atomic_axpy_col<R>(scatter_target(B, shadow.b, wp, slot, d), scale_of(wp, vexp, smode), dbb,
-                         lane, d);
+      atomic_axpy_col<R>(scatter_ref(tables.b(wp, d), shadow.b, slot, d),
+                         scale_of(wp, vexp, smode), dbb, lane, d);
     }
     __syncthreads();
   }
@@ -439,16 +462,19 @@ static int pick_tile(int R, int Sh) {
   return T;
 }
 
-template <int R>
+// Launches the tiled pass and the fold of the shadow copies into fold_a / fold_b (the tables that
+// hold the shadowed columns).  *launched is false, and nothing is enqueued, if no tile fits.
+template <int R, class Tables>
 static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int shift, const int* W,
-                                    const int* LB, const int* UB, float* A, float* B, float lrate,
-                                    float vexp, Shadow shadow) {
+                                    const int* LB, const int* UB, const Tables& tables,
+                                    float* fold_a, float* fold_b, float lrate, float vexp,
+                                    Shadow shadow, bool* launched) {
   const int Sh = shift < 0 ? 0 : (shift > kMaxHalo ? kMaxHalo : shift);
   const int T = Sh > 0 ? pick_tile(R, Sh) : 0;
-  if (T == 0)
-    return launch_pos_r<R, true>(stream, d, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr);
+  *launched = T != 0;
+  if (T == 0) return hipSuccess;
   const size_t lds = tile_lds_bytes(R, T, Sh);
-  auto kern = pos_tile_kernel<R>;
+  auto kern = pos_tile_kernel<R, Tables>;
   hipError_t err = hipSuccess;
   if (lds > 48 * 1024) {
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -463,10 +489,22 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
   nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
-                     ntiles, tiles_per_wg, W, LB, UB, A, B, lrate, vexp, scale_mode(vexp), shadow);
+                     ntiles, tiles_per_wg, W, LB, UB, tables, lrate, vexp, scale_mode(vexp),
+                     shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
-  return launch_fold(stream, A, B, shadow, d);
+  return launch_fold(stream, fold_a, fold_b, shadow, d);
+}
+
+template <int R>
+static hipError_t launch_pos_plain_r(hipStream_t stream, int d, int ncols, int shift, const int* W,
+                                     const int* LB, const int* UB, float* A, float* B, float lrate,
+                                     float vexp, Shadow shadow) {
+  bool launched = false;
+  hipError_t err = launch_pos_tile_r<R>(stream, d, ncols, shift, W, LB, UB, PlainTables{A, B}, A, B,
+                                        lrate, vexp, shadow, &launched);
+  if (err != hipSuccess || launched) return err;
+  return launch_pos_r<R, true>(stream, d, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr);
 }
 
 hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
@@ -474,7 +512,18 @@ hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const
                       Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R) \
-  return launch_pos_tile_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, shadow)
+  return launch_pos_plain_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, shadow)
+  W2V_ROUNDS_SWITCH(rounds, CALL)
+#undef CALL
+}
+
+hipError_t launch_slice_pos_tiled(hipStream_t stream, int nrows, int ncols, int shift,
+                                  const int* W, const int* LB, const int* UB, const SliceMap& m,
+                                  float lrate, float vexp, Shadow shadow, bool* launched) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+#define CALL(R)                                                                                 \
+  return launch_pos_tile_r<R>(stream, nrows, ncols, shift, W, LB, UB, SlicedTables{m}, m.mats[1], \
+                              m.mats[0], lrate, vexp, shadow, launched)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }

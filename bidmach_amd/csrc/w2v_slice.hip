@@ -16,37 +16,17 @@
 //   (so head columns can be trained by one designated worker, or by all of them and averaged).
 // Rule of the forward pass: a pair is scored iff both words are resident.
 //
-// With a model of several hundred gigabytes in mind the kernels are the plain wave-per-unit
-// forms (one wavefront per centre token / per group, columns in registers, one column of line-
-// aligned float atomics per written column), persistent over contiguous ranges of work units so
-// that the work in flight is bounded the same way as in the single-table passes.
+// The positive update runs through the tiled kernel of the single-table pass (w2v_pos.hip), which
+// takes the model as a policy; the kernels here are the negative update, the forward-only twins,
+// and the per-centre positive update used when no tile fits in LDS.  All are wave-per-unit
+// (columns in registers, one column of line-aligned float atomics per written column) and
+// persistent over contiguous ranges of work units, so the work in flight is bounded the same
+// way as in the single-table passes.  The first kHotWords packed columns of part 0 (the most
+// frequent head words) are read and updated through their shadow copies during an update.
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
 namespace w2v {
-
-constexpr int kMine = 1;  // the worker's own tail word
-constexpr int kHead = 2;  // head word, resident on every worker
-
-struct Placed {
-  float* col;  // start of the word's column, null if the word is not resident
-  int flags;   // 0 (not resident), kMine or kHead
-};
-
-// which: 0 = B table of the part, 1 = A table.
-__device__ __forceinline__ Placed place(const SliceMap& m, int w, int which, int d) {
-  Placed p{nullptr, 0};
-  if (w < 0) return p;
-  const bool head = w < m.nhead;
-  const bool mine = !head && (w % m.nslices == m.islice);
-  if (!head && !mine) return p;
-  const int packed = head ? w : (w - m.nhead) / m.nslices + m.nhead;
-  const int part = packed / m.maxcols;
-  if (part >= m.nparts) return p;
-  p.col = m.mats[2 * part + which] + (int64_t)(packed - part * m.maxcols) * d;
-  p.flags = head ? kHead : kMine;
-  return p;
-}
 
 __device__ __forceinline__ float* read_lane_ptr(float* p, int lane) {
   const uint64_t v = reinterpret_cast<uint64_t>(p);
@@ -55,22 +35,26 @@ __device__ __forceinline__ float* read_lane_ptr(float* p, int lane) {
   return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
 }
 
-// Both flags non-zero (both words resident) is tested by the callers.
-__device__ __forceinline__ bool pair_trained(int fa, int fb, int dohead) {
-  return (((fa | fb) & kMine) != 0) || dohead > 1;
+__device__ __forceinline__ ColRef read_lane_ref(const ColRef& r, int lane) {
+  return ColRef{read_lane_ptr(r.col, lane), read_lane(r.hot, lane), read_lane(r.flags, lane)};
 }
 
-__device__ __forceinline__ bool col_written(int f, int dohead) {
-  return f == kMine || (f == kHead && dohead > 0);
+// The forward-only kernels never see non-zero shadows (they are zero between update calls).
+template <bool TRAIN>
+__device__ __forceinline__ ColRef for_pass(ColRef r) {
+  if (!TRAIN) r.hot = -1;
+  return r;
 }
 
 template <int R, int CH, bool TRAIN>
 __global__ void __launch_bounds__(kBlock)
 slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ W,
-                 const int* __restrict__ LB, const int* __restrict__ UB, SliceMap m, float lrate,
-                 float vexp, int smode, double floorv, double* __restrict__ partials) {
+                 const int* __restrict__ LB, const int* __restrict__ UB, SlicedTables tables,
+                 float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
+                 Shadow shadow) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slot = blockIdx.x;
   const int64_t u_begin = (int64_t)blockIdx.x * units_per_wg;
   const int64_t u_end = min(u_begin + units_per_wg, (int64_t)ncols);
   double lsum = 0.0;
@@ -78,12 +62,12 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
   for (int64_t unit = u_begin + wave; unit < u_end; unit += kWavesPerBlock) {
     const int i = (int)unit;
     const int wi = __builtin_amdgcn_readfirstlane(W[i]);
-    const Placed pa = place(m, wi, 1, d);
+    const ColRef pa = for_pass<TRAIN>(tables.a(wi, d));
     if (pa.flags == 0) continue;
     const int jlo = max(LB[i], -i);
     const int jhi = min(UB[i], ncols - 1 - i);
     float a[R];
-    load_col<R>(a, pa.col, lane, d);
+    load_col_ref<R>(a, pa, shadow.a, lane, d);
     float daa[R];
     zero_col<R>(daa);
     const float ascale = TRAIN ? scale_of(wi, vexp, smode) : 1.0f;
@@ -93,12 +77,12 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
       const int j = base + lane;
       int wl = -1;
       if (j <= jhi && j != 0) wl = W[i + j];
-      const Placed pb = place(m, wl, 0, d);
+      const ColRef pb = for_pass<TRAIN>(tables.b(wl, d));
       bool ok = pb.flags != 0;
-      if (TRAIN) ok = ok && pair_trained(pa.flags, pb.flags, m.dohead);
+      if (TRAIN) ok = ok && tables.trained(pa.flags, pb.flags);
       const float sl = (TRAIN && ok) ? scale_of(wl, vexp, smode) : 0.0f;
       unsigned long long mask = __ballot(ok);
-      const unsigned long long wmask = __ballot(ok && col_written(pb.flags, m.dohead));
+      const unsigned long long wmask = __ballot(ok && tables.written(pb.flags));
 
       while (mask != 0ull) {
         int src[CH];
@@ -114,12 +98,12 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
           }
         }
         float b[CH][R];
-        float* bcol[CH];
+        ColRef rb[CH];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
           if (c < n) {
-            bcol[c] = read_lane_ptr(pb.col, src[c]);
-            load_col<R>(b[c], bcol[c], lane, d);
+            rb[c] = read_lane_ref(pb, src[c]);
+            load_col_ref<R>(b[c], rb[c], shadow.b, lane, d);
           }
         }
         float pre = 0.0f;
@@ -139,7 +123,8 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
               const float g = read_lane(gl, c);
               const float bs = read_lane(sl, src[c]);
               axpy<R>(daa, ascale * g, b[c]);
-              if ((wmask >> src[c]) & 1ull) atomic_axpy_col<R>(bcol[c], bs * g, a, lane, d);
+              if ((wmask >> src[c]) & 1ull)
+                atomic_axpy_col<R>(scatter_ref(rb[c], shadow.b, slot, d), bs * g, a, lane, d);
             }
           }
           touched = true;
@@ -148,21 +133,23 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
         }
       }
     }
-    if (TRAIN && touched && col_written(pa.flags, m.dohead))
-      atomic_add_col<R>(pa.col, daa, lane, d);
+    if (TRAIN && touched && tables.written(pa.flags))
+      atomic_add_col<R>(scatter_ref(pa, shadow.a, slot, d), daa, lane, d);
   }
 
   if (!TRAIN) block_store_partial(wave_sum_f64(lsum), partials);
 }
 
 template <int R, int MAXB, int CHA, bool TRAIN>
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kBlock, 3)
 slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
-                 const int* __restrict__ WA, const int* __restrict__ WB, SliceMap m, float lrate,
-                 float vexp, int smode, double floorv, double* __restrict__ partials) {
+                 const int* __restrict__ WA, const int* __restrict__ WB, SlicedTables tables,
+                 float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
+                 Shadow shadow) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slot = blockIdx.x;
   const int64_t u_begin = (int64_t)blockIdx.x * units_per_wg;
   const int64_t u_end = min(u_begin + units_per_wg, (int64_t)ngroups);
   double lsum = 0.0;
@@ -170,21 +157,21 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
   for (int64_t unit = u_begin + wave; unit < u_end; unit += kWavesPerBlock) {
     int wbl = -1;
     if (lane < nwb) wbl = WB[unit * nwb + lane];
-    const Placed pbl = place(m, wbl, 0, d);
+    const ColRef pbl = for_pass<TRAIN>(tables.b(wbl, d));
     const float sbl = (TRAIN && pbl.flags != 0) ? scale_of(wbl, vexp, smode) : 0.0f;
 
     float b[MAXB][R];
     float dbb[MAXB][R];
-    float* bcol[MAXB];
+    ColRef rb[MAXB];
     int fb[MAXB];
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       fb[k] = 0;
-      bcol[k] = nullptr;
+      rb[k] = ColRef{nullptr, -1, 0};
       if (k < nwb) {
-        fb[k] = read_lane(pbl.flags, k);
-        bcol[k] = read_lane_ptr(pbl.col, k);
-        if (fb[k] != 0) load_col<R>(b[k], bcol[k], lane, d);
+        rb[k] = read_lane_ref(pbl, k);
+        fb[k] = rb[k].flags;
+        if (fb[k] != 0) load_col_ref<R>(b[k], rb[k], shadow.b, lane, d);
         zero_col<R>(dbb[k]);
       }
     }
@@ -192,22 +179,22 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
       int wal = -1;
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
-      const Placed pal = place(m, wal, 1, d);
+      const ColRef pal = for_pass<TRAIN>(tables.a(wal, d));
       const float sal = (TRAIN && pal.flags != 0) ? scale_of(wal, vexp, smode) : 0.0f;
       const int jend = min(nwa - jbase, kWave);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
         float a[CHA][R];
-        float* acol[CHA];
+        ColRef ra[CHA];
         int fa[CHA];
 #pragma unroll
         for (int c = 0; c < CHA; ++c) {
           fa[c] = 0;
-          acol[c] = nullptr;
+          ra[c] = ColRef{nullptr, -1, 0};
           if (j0 + c < jend) {
-            fa[c] = read_lane(pal.flags, j0 + c);
-            acol[c] = read_lane_ptr(pal.col, j0 + c);
-            if (fa[c] != 0) load_col<R>(a[c], acol[c], lane, d);
+            ra[c] = read_lane_ref(pal, j0 + c);
+            fa[c] = ra[c].flags;
+            if (fa[c] != 0) load_col_ref<R>(a[c], ra[c], shadow.a, lane, d);
           }
         }
         float pre = 0.0f;
@@ -217,7 +204,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
           if (fa[c] != 0) {
 #pragma unroll
             for (int k = 0; k < MAXB; ++k) {
-              if (fb[k] != 0 && (!TRAIN || pair_trained(fa[c], fb[k], m.dohead))) {
+              if (fb[k] != 0 && (!TRAIN || tables.trained(fa[c], fb[k]))) {
                 const float s = wave_sum(dot_partial<R>(a[c], b[k]));
                 const bool here = lane == c * MAXB + k;
                 pre = here ? s : pre;
@@ -236,14 +223,15 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
               zero_col<R>(daa);
 #pragma unroll
               for (int k = 0; k < MAXB; ++k) {
-                if (fb[k] != 0 && pair_trained(fa[c], fb[k], m.dohead)) {
+                if (fb[k] != 0 && tables.trained(fa[c], fb[k])) {
                   const float g = read_lane(gl, c * MAXB + k);
                   const float bs = read_lane(sbl, k);
                   axpy<R>(dbb[k], bs * g, a[c]);
                   axpy<R>(daa, as * g, b[k]);
                 }
               }
-              if (col_written(fa[c], m.dohead)) atomic_add_col<R>(acol[c], daa, lane, d);
+              if (tables.written(fa[c]))
+                atomic_add_col<R>(scatter_ref(ra[c], shadow.a, slot, d), daa, lane, d);
             }
           }
         } else {
@@ -255,8 +243,8 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     if (TRAIN) {
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
-        if (fb[k] != 0 && col_written(fb[k], m.dohead))
-          atomic_add_col<R>(bcol[k], dbb[k], lane, d);
+        if (fb[k] != 0 && tables.written(fb[k]))
+          atomic_add_col<R>(scatter_ref(rb[k], shadow.b, slot, d), dbb[k], lane, d);
       }
     }
   }
@@ -295,13 +283,14 @@ static hipError_t slice_grid(const void* kernel, int64_t units, int64_t* nwg, in
 template <int R, bool TRAIN>
 static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const int* W,
                                      const int* LB, const int* UB, const SliceMap& m, float lrate,
-                                     float vexp, double floorv, double* partials, int64_t* nparts) {
+                                     float vexp, double floorv, double* partials, int64_t* nparts,
+                                     Shadow shadow) {
   auto kern = slice_pos_kernel<R, SlicePosChunk<R>::value, TRAIN>;
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ncols, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
-                     UB, m, lrate, vexp, scale_mode(vexp), floorv, partials);
+                     UB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials, shadow);
   *nparts = nwg;
   return hipGetLastError();
 }
@@ -310,13 +299,14 @@ template <int R, int MAXB, bool TRAIN>
 static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
                                       const int* WA, const int* WB, const SliceMap& m, float lrate,
                                       float vexp, double floorv, double* partials,
-                                      int64_t* nparts) {
+                                      int64_t* nparts, Shadow shadow) {
   auto kern = slice_neg_kernel<R, MAXB, SliceNegChunk<R, MAXB>::value, TRAIN>;
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ngroups, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
-                     per_wg, WA, WB, m, lrate, vexp, scale_mode(vexp), floorv, partials);
+                     per_wg, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials,
+                     shadow);
   *nparts = nwg;
   return hipGetLastError();
 }
@@ -324,37 +314,50 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
 template <int R, bool TRAIN>
 static hipError_t launch_slice_neg_r(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
                                      const int* WA, const int* WB, const SliceMap& m, float lrate,
-                                     float vexp, double floorv, double* partials, int64_t* nparts) {
+                                     float vexp, double floorv, double* partials, int64_t* nparts,
+                                     Shadow shadow) {
   if (nwb <= 5)
     return launch_slice_neg_rb<R, 5, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
-                                            floorv, partials, nparts);
+                                            floorv, partials, nparts, shadow);
   if (nwb <= 8)
     return launch_slice_neg_rb<R, 8, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
-                                            floorv, partials, nparts);
+                                            floorv, partials, nparts, shadow);
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                            const int* UB, const SliceMap& m, float lrate, float vexp) {
+hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                            const int* LB, const int* UB, const SliceMap& m, float lrate,
+                            float vexp, Shadow shadow) {
+  bool launched = false;
+  hipError_t err = launch_slice_pos_tiled(stream, nrows, ncols, shift, W, LB, UB, m, lrate, vexp,
+                                          shadow, &launched);
+  if (err != hipSuccess || launched) return err;
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
-#define CALL(R)                                                                                 \
-  return launch_slice_pos_r<R, true>(stream, nrows, ncols, W, LB, UB, m, lrate, vexp, 0.0, nullptr, \
-                                     &unused)
+#define CALL(R)                                                                               \
+  err = launch_slice_pos_r<R, true>(stream, nrows, ncols, W, LB, UB, m, lrate, vexp, 0.0, nullptr, \
+                                    &unused, shadow);                                         \
+  break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
+  if (err != hipSuccess) return err;
+  return launch_fold(stream, m.mats[1], m.mats[0], shadow, nrows);
 }
 
 hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                             const int* WA, const int* WB, const SliceMap& m, float lrate,
-                            float vexp) {
+                            float vexp, Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
-#define CALL(R)                                                                               \
-  return launch_slice_neg_r<R, true>(stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate, vexp, 0.0, \
-                                     nullptr, &unused)
+  hipError_t err = hipSuccess;
+#define CALL(R)                                                                                \
+  err = launch_slice_neg_r<R, true>(stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate, vexp, 0.0, \
+                                    nullptr, &unused, shadow);                                 \
+  break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
+  if (err != hipSuccess) return err;
+  return launch_fold(stream, m.mats[1], m.mats[0], shadow, nrows);
 }
 
 hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const int* W,
@@ -365,7 +368,7 @@ hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const
   int64_t nparts = 0;
 #define CALL(R)                                                                                   \
   err = launch_slice_pos_r<R, false>(stream, nrows, ncols, W, LB, UB, m, 0.0f, 0.0f, floorv,      \
-                                     partials, &nparts);                                          \
+                                     partials, &nparts, Shadow{});                                \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
@@ -381,7 +384,7 @@ hipError_t launch_slice_eval_neg(hipStream_t stream, int nrows, int ncols, int n
   int64_t nparts = 0;
 #define CALL(R)                                                                                   \
   err = launch_slice_neg_r<R, false>(stream, nrows, ncols, nwa, nwb, WA, WB, m, 0.0f, 0.0f,       \
-                                     floorv, partials, &nparts);                                  \
+                                     floorv, partials, &nparts, Shadow{});                        \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL

@@ -155,6 +155,25 @@ def test_eval_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols,
     assert got[1] == pytest.approx(wneg, rel=EVAL_RTOL)
 
 
+@pytest.mark.parametrize("shift", [0, 1, 40])
+def test_pos_slice_result_does_not_depend_on_shift(gpu, oracle, shift):
+    """`shift` only sizes the halo staged on chip: 0 takes the per-centre kernel, 1 leaves most of
+    the window to the gather path of the tiled kernel, 40 is clamped."""
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(17)
+    V, d, skip = 2600, 100, 4
+    islice, nslices, nhead, maxcols, dohead = 1, 2, 200, 500, 1
+    A, B = rand_tables(rng, V, d, 0.15)
+    W, LB, UB = corpus.collision_free_pos(280, skip, V, rng)
+    host, devl = model_lists(torch, A, B, islice, nslices, nhead, maxcols, False)
+    oracle.word2vecPosSlice(d, len(W), skip, W, LB, UB, host, 0.05, 0.0, 1, islice, nslices,
+                            maxcols, nhead, 0, dohead)
+    err = CUMACH.word2vecPosSlice(d, len(W), shift, dev(torch, W), dev(torch, LB), dev(torch, UB),
+                                  devl, 0.05, 0.0, islice, nslices, maxcols, nhead, 0, dohead)
+    assert err == 0
+    assert_lists_close(devl, host, UPDATE_ATOL)
+
+
 def test_colliding_minibatch_stays_close_to_sequential_oracle(gpu, oracle):
     """A Zipf minibatch on a three-part, two-worker model with a small step: the Hogwild result
     differs from the single-thread oracle only in second order."""
