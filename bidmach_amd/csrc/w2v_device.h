@@ -174,33 +174,6 @@ struct Shadow {
   float* b;  // same for table B
 };
 
-template <int R>
-__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
-                                             const float* shadow, int w, int lane, int d) {
-  load_col<R>(x, table + (int64_t)w * d, lane, d);
-  if (w < kHotWords) {
-    // two shadow copies per trip: enough loads in flight without inflating the register count
-    // of the callers, which inline this many times
-    const int copies = shadow_copies(w);
-#pragma unroll 1
-    for (int s = 0; s < copies; s += 2) {
-      float y0[R], y1[R];
-      load_col<R>(y0, shadow + ((int64_t)s * kHotWords + w) * d, lane, d);
-      load_col<R>(y1, shadow + ((int64_t)(s + 1) * kHotWords + w) * d, lane, d);
-#pragma unroll
-      for (int r = 0; r < R; ++r) x[r] += y0[r] + y1[r];
-    }
-  }
-}
-
-// Column that receives the atomics for word w from workgroup number `wg`.
-__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int wg,
-                                                 int d) {
-  if (w >= kHotWords) return table + (int64_t)w * d;
-  const int slot = wg & (shadow_copies(w) - 1);
-  return shadow + ((int64_t)slot * kHotWords + w) * d;
-}
-
 // ---- where a word's column lives -------------------------------------------------------------
 //
 // The kernels that serve both the single-table model and the sliced, multi-part model see the
@@ -238,6 +211,22 @@ __device__ __forceinline__ float* scatter_ref(const ColRef& ref, float* shadow, 
   if (ref.hot < 0) return ref.col;
   const int slot = wg & (shadow_copies(ref.hot) - 1);
   return shadow + ((int64_t)slot * kHotWords + ref.hot) * d;
+}
+
+// A table-relative form of the two helpers above, for kernels that address one pair of tables by
+// word id: column w of `table`, shadowed iff w < kHotWords.
+template <int R>
+__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
+                                             const float* shadow, int w, int lane, int d) {
+  const ColRef ref{const_cast<float*>(table) + (int64_t)w * d, w < kHotWords ? w : -1, kMine};
+  load_col_ref<R>(x, ref, shadow, lane, d);
+}
+
+// Column that receives the atomics for word w from workgroup number `wg`.
+__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int wg,
+                                                 int d) {
+  const ColRef ref{table + (int64_t)w * d, w < kHotWords ? w : -1, kMine};
+  return scatter_ref(ref, shadow, wg, d);
 }
 
 // One pair of tables: word w is column w of A / of B; every pair is trained, every column written.
