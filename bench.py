@@ -114,6 +114,11 @@ def main():
     ap.add_argument("--parts", type=int, default=0,
                     help="train mode only: cut each table into this many separate allocations and "
                          "run the step through word2vecPosSlice + word2vecNegSlice (one worker)")
+    ap.add_argument("--slices", type=int, default=1,
+                    help="with --parts: number of workers the tail of the vocabulary is dealt to; "
+                         "this process is worker 0 and holds only its share of the model")
+    ap.add_argument("--head", type=int, default=0,
+                    help="with --parts: number of head words (resident on every worker)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -162,10 +167,16 @@ def main():
     ret = torch.zeros(2, dtype=torch.float32, device="cuda")
     MM, maxcols = None, 0
     if args.parts > 0 and not evaluating:
-        maxcols = (V + args.parts - 1) // args.parts
+        # worker 0 of --slices: head words, then its tail words in id order, cut into --parts parts
+        ids = torch.arange(V, device="cuda")
+        keep = (ids < args.head) | ((ids >= args.head) & (ids % args.slices == 0))
+        packedB, packedA = B[keep], A[keep]
+        resident = packedB.shape[0]
+        maxcols = (resident + args.parts - 1) // args.parts
         MM = []
-        for c0 in range(0, V, maxcols):
-            MM += [B[c0:c0 + maxcols].clone(), A[c0:c0 + maxcols].clone()]
+        for c0 in range(0, resident, maxcols):
+            MM += [packedB[c0:c0 + maxcols].clone(), packedA[c0:c0 + maxcols].clone()]
+        del ids, keep, packedA, packedB
 
     def step(s, timers=None):
         mb, hmb = dev_mbs[s % ndistinct], host_mbs[s % ndistinct]
@@ -177,7 +188,7 @@ def main():
                                               ret[0:1]), "word2vecEvalPos")
         elif MM:
             check(CUMACH.word2vecPosSlice(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], MM, lr,
-                                          args.vexp, 0, 1, maxcols, 0, False, 1),
+                                          args.vexp, 0, args.slices, maxcols, args.head, False, 1),
                   "word2vecPosSlice")
         else:
             check(CUMACH.word2vecPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr,
@@ -190,8 +201,8 @@ def main():
                                               mb["WB"], A, B, ret[1:2]), "word2vecEvalNeg")
         elif MM:
             check(CUMACH.word2vecNegSlice(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
-                                          mb["WB"], MM, lr / cfg["nneg"], args.vexp, 0, 1, maxcols,
-                                          0, False, 1), "word2vecNegSlice")
+                                          mb["WB"], MM, lr / cfg["nneg"], args.vexp, 0, args.slices,
+                                          maxcols, args.head, False, 1), "word2vecNegSlice")
         else:
             check(CUMACH.word2vecNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                           mb["WB"], A, B, lr / cfg["nneg"], args.vexp),
@@ -279,6 +290,8 @@ def main():
         out["roofline"]["traffic"] = None
     if MM:
         out["config"]["parts"] = len(MM) // 2
+        out["config"]["slices"] = args.slices
+        out["config"]["head_words"] = args.head
         out["config"]["operators"] = "word2vecPosSlice+word2vecNegSlice"
         out["roofline"]["traffic"] = None
     if not evaluating and not MM and not args.no_pcie:
