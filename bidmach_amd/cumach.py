@@ -74,6 +74,9 @@ SYMBOLS = {
     "w2v_timer_stop": (_I, [_P]),
     "w2v_timer_elapsed_ms": (_I, [_P, ctypes.POINTER(_F)]),
     "w2v_error_string": (ctypes.c_char_p, [_I]),
+    "w2v_lz4_compress_bound": (_SZ, [_SZ]),
+    "w2v_lz4_compress": (ctypes.c_longlong, [_P, _SZ, _P, _SZ]),
+    "w2v_lz4_decompress": (ctypes.c_longlong, [_P, _SZ, _P, _SZ]),
 }
 
 

@@ -16,6 +16,9 @@ What is mirrored (src/main/scala/BIDMach/networks/Word2Vec.scala of the referenc
                   operators when nSlices != 1 or the model needs more than one part (:178-187,
                   :196-207).  The reference runs those on the CPU only; here every part is a
                   device allocation and the library's device Slice operators are used.
+  save / load     the checkpoint layout of Model.save / Model.load (models/Model.scala:245-315):
+                  `options.json` and one `modelmat%02d.lz4` per model matrix under a path prefix
+                  (the Java-serialised `options.ser` is not written)
   train           Learner.nextPass' loop: minibatch istep is scored instead of trained on when
                   (istep - 1) % evalStep == 0, and so is the last one of a pass
                   (Learner.scala:187-222, evalStep default 11 at :1064)
@@ -280,6 +283,45 @@ class Word2Vec:
             eneg = self.evalNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
                                       self.modelmats[0])
         return (epos + eneg / (1 if o.eqPosNeg else o.nneg)) / goodwords.shape[0]
+
+    # ---- Model.save / Model.load (models/Model.scala:245-315) ---------------------------
+    def save(self, fname):
+        """Writes `fname + "options.json"` and `fname + "modelmat%02d.lz4"` for every model matrix
+        (BIDMat dense-matrix files, dim x columns, LZ4 block stream).  `fname` is a path prefix,
+        normally a directory name ending in a separator, created if needed."""
+        import json
+        import os
+        from . import matio
+        parent = os.path.dirname(fname + "options.json")
+        if parent:
+            os.makedirs(parent, exist_ok=True)
+        with open(fname + "options.json", "w") as f:
+            json.dump({k: v for k, v in vars(self.opts).items()}, f, indent=1, sort_keys=True)
+        for i, m in enumerate(self.modelmats):
+            matio.saveMat(fname + "modelmat%02d.lz4" % i, m.cpu().numpy().T)
+
+    def load(self, fname, useJson=True):
+        """Reads the model matrices `fname + "modelmat%02d.lz4"` (as many as exist) and, with
+        useJson, the options; a model loaded this way is not re-initialised (`refresh = false`,
+        Model.scala:314)."""
+        import json
+        import os
+        from . import matio
+        if useJson and os.path.exists(fname + "options.json"):
+            with open(fname + "options.json") as f:
+                for k, v in json.load(f).items():
+                    if hasattr(self.opts, k):
+                        setattr(self.opts, k, v)
+        mats = []
+        while os.path.exists(fname + "modelmat%02d.lz4" % len(mats)):
+            m = matio.loadFMat(fname + "modelmat%02d.lz4" % len(mats))
+            if m.shape[0] != self.opts.dim:
+                raise ValueError("modelmat%02d has %d rows, the model's dim is %d"
+                                 % (len(mats), m.shape[0], self.opts.dim))
+            mats.append(np.array(m.T, order="C", copy=True))     # loadMat's buffer is read-only
+        if len(mats) < 2 or len(mats) % 2:
+            raise ValueError("no model matrices under %r" % fname)
+        self.init(self.ncols, modelmats=mats)
 
     # ---- Learner.nextPass, reduced to what Word2Vec uses (no updater, no mixins) ---------
     def train(self, stream, npasses=1):

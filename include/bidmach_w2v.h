@@ -174,6 +174,16 @@ int w2v_timer_elapsed_ms(void *timer, float *ms); /* waits for the stop event */
 /* Text of an error code returned by any function above. */
 const char *w2v_error_string(int err);
 
+/* LZ4 block codec on HOST memory, for the reference's on-disk files either side of the path:
+ * model checkpoints `modelmat%02d.lz4` (Model.scala:259-262, :284-292) and `.imat.lz4` word files.
+ * It stands in for the codec BIDMat reaches through lz4-java (both out of the reference tree) and
+ * implements the published LZ4 block format; the stream framing is done by the caller.
+ * compress/decompress return the number of bytes written, or -1 (output too small, or malformed
+ * input); w2v_lz4_compress_bound(n) bytes of output always suffice to compress n bytes. */
+size_t w2v_lz4_compress_bound(size_t n);
+long long w2v_lz4_compress(const void *src, size_t n, void *dst, size_t capacity);
+long long w2v_lz4_decompress(const void *src, size_t n, void *dst, size_t capacity);
+
 #ifdef __cplusplus
 }
 #endif
