@@ -151,3 +151,31 @@ def test_sliced_multipart_model_matches_oracle_step(oracle, dual):
     want = (epos + eneg / o.nneg) / ctx.shape[0]
     assert want < -0.05
     assert got == pytest.approx(want, rel=1e-5)
+
+
+def test_train_from_word_file_then_checkpoint_round_trip(tmp_path):
+    """The files either side of the path: a (word id, sentence id) .imat.lz4 input file feeds the
+    training loop, the model is written in the checkpoint layout, and a fresh model loaded from it
+    scores a held-out minibatch identically."""
+    import os
+    from bidmach_amd import matio
+    words = str(tmp_path / "words.imat.lz4")
+    matio.saveIMat(words, make_stream(4000 * 6, 3000, seed=31))
+    o = Options(vocabSize=3000, dim=32, batchSize=4000, lrate=0.05, evalStep=100, seed=6)
+    m = Word2Vec(o)
+    res = m.train(matio.loadIMat(words), npasses=1)
+    assert len(res) == 2 and all(np.isfinite(r[1]) for r in res)    # minibatch 1 and the last one
+    prefix = str(tmp_path / "model") + os.sep
+    m.save(prefix)
+    m2 = Word2Vec(Options(dim=32, batchSize=4000))
+    m2.load(prefix)
+    m2.ncols = 4000
+    for a, b in zip(m.modelmats, m2.modelmats):
+        assert a.is_cuda and b.is_cuda and bool((a == b).all())
+    held = make_stream(4000, 3000, seed=32)
+    m.rng = np.random.Generator(np.random.PCG64(1))
+    m2.rng = np.random.Generator(np.random.PCG64(1))
+    m._call = m2._call = 1000
+    s1 = m.evalbatch(held, 0, 4000)
+    s2 = m2.evalbatch(held, 0, 4000)
+    assert s1 < -0.1 and s1 == s2
