@@ -43,12 +43,14 @@ WORKLOADS = {
 }
 
 
-def make_minibatch(cfg, index, zcdf, ncdf):
+def make_minibatch(cfg, index, zcdf, ncdf, wsample=0.0):
     """Index arrays of minibatch `index` of the stream (seeded, reproducible)."""
     from bidmach_amd import corpus
     n = cfg["tokens"]
     W = corpus.zipf_stream(n, cfg["vocab"], cfg["zipf"], seed=1234 + index, cdf=zcdf)
     rng = np.random.Generator(np.random.PCG64(99 + index))
+    if wsample > 0.0:       # the reference caller's frequent-word subsampling: dropped words are -1
+        W = corpus.subsample(W, cfg["vocab"], wsample, rng)
     LB, UB = corpus.window_bounds(n, cfg["skip"], rng)
     WA, WB, G = corpus.negative_groups(W, LB, UB, cfg["nneg"], cfg["nreuse"], rng, neg_cdf=ncdf)
     pairs, centres = corpus.count_pairs(W, LB, UB)
@@ -119,6 +121,9 @@ def main():
                          "this process is worker 0 and holds only its share of the model")
     ap.add_argument("--head", type=int, default=0,
                     help="with --parts: number of head words (resident on every worker)")
+    ap.add_argument("--wsample", type=float, default=0.0,
+                    help="frequent-word subsampling threshold of the reference caller (its default "
+                         "is 1e-4); 0 = the raw stream the headline metric is defined on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -144,7 +149,7 @@ def main():
     zcdf = corpus.zipf_cdf(V, cfg["zipf"])
     ncdf = corpus.unigram_pow_cdf(V, cfg["zipf"], 0.75)
     ndistinct = max(1, min(args.distinct, K + Wm))
-    host_mbs = [make_minibatch(cfg, i, zcdf, ncdf) for i in range(ndistinct)]
+    host_mbs = [make_minibatch(cfg, i, zcdf, ncdf, args.wsample) for i in range(ndistinct)]
     dev_mbs = []
     for mb in host_mbs:
         dev_mbs.append({k: torch.from_numpy(mb[k]).cuda() for k in ("W", "LB", "UB", "WA", "WB")})
@@ -287,6 +292,9 @@ def main():
 
     if evaluating:
         out["config"]["mode"] = "eval"
+        out["roofline"]["traffic"] = None
+    if args.wsample > 0.0:
+        out["config"]["wsample"] = args.wsample
         out["roofline"]["traffic"] = None
     if MM:
         out["config"]["parts"] = len(MM) // 2
