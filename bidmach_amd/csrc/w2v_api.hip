@@ -52,7 +52,8 @@ hipError_t eval_scratch(int64_t need, double** out) {
   return hipSuccess;
 }
 
-// Per-thread, per-device shadow buffers for the hot columns, allocated and zeroed on first use.
+// Per-thread, per-device shadow buffers for the hot columns and their write counters, allocated
+// and zeroed on first use: [shadow of A | shadow of B | counters].
 hipError_t shadow_buffers(w2v::Shadow* out) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -62,9 +63,10 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   const size_t bytes = w2v::shadow_bytes();
   if (ts.shadow[dev] == nullptr) {
     float* p = nullptr;
-    err = hipMalloc(reinterpret_cast<void**>(&p), 2 * bytes);
+    const size_t total = 2 * bytes + w2v::shadow_counter_bytes();
+    err = hipMalloc(reinterpret_cast<void**>(&p), total);
     if (err != hipSuccess) return err;
-    err = hipMemsetAsync(p, 0, 2 * bytes, ts.stream);
+    err = hipMemsetAsync(p, 0, total, ts.stream);
     if (err == hipSuccess) err = hipStreamSynchronize(ts.stream);  // the stream may change later
     if (err != hipSuccess) {
       (void)hipFree(p);
@@ -74,6 +76,8 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   }
   out->a = ts.shadow[dev];
   out->b = ts.shadow[dev] + bytes / sizeof(float);
+  out->count = reinterpret_cast<unsigned*>(ts.shadow[dev] + 2 * (bytes / sizeof(float)));
+  out->combine = 0;
   return hipSuccess;
 }
 
@@ -352,6 +356,12 @@ int w2v_set_max_workgroups(int n) {
   return 0;
 }
 int w2v_get_max_workgroups(void) { return w2v::get_max_workgroups(); }
+
+int w2v_set_hot_update_mode(int mode) {
+  w2v::set_hot_update_mode(mode);
+  return 0;
+}
+int w2v_get_hot_update_mode(void) { return w2v::get_hot_update_mode(); }
 
 int w2v_max_rows(void) { return w2v::max_rows(); }
 int w2v_max_nwb(void) { return w2v::max_nwb(); }

@@ -151,28 +151,47 @@ __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float a
 
 // Shadow copies of the hottest columns.
 //
-// Word ids are frequency ranks, so under a Zipf law ids 0..7 each receive hundreds of thousands
-// of column updates per call.  Atomics to one cache line retire one after the other in L2
-// (about 36 ns each), which would make those few columns the critical path of the whole pass.
-// While a pass runs, the value of a hot column w < kHotWords is therefore represented as
-//     table[w] + sum over s < kShadows of shadow[s][w]
-// with the shadows in a scratch buffer that is zero between calls: a reader sums all copies, a
-// writer adds into the one copy chosen by its workgroup index, so the same-line queue is spread
-// over several lines and no update is delayed or dropped.  A small kernel folds the shadows
-// back into the table (and zeroes them) at the end of the call.  The number of copies follows
-// the Zipf law: 16 for word 0, 8 for words 1-2, 4 for words 3-6, 2 for word 7, so every hot
-// line sees about the same queue and readers do not sum more copies than needed.
-constexpr int kHotWords = 8;
-constexpr int kShadows = 16;
+// Word ids are frequency ranks, so under a Zipf law the first few ids each receive hundreds of
+// thousands of column updates per call.  Atomics to one cache line retire one after the other in
+// L2 (about 36 ns each), and reads of that line queue behind them, which would make those few
+// columns the critical path of the whole pass.  The atomics for a hot column therefore go to one
+// of several shadow copies of it (chosen by the workgroup index) in a scratch buffer that is zero
+// between calls, so the same-line queue is spread over several lines.  A small kernel moves what
+// is left in the copies into the table at the end of the call.  Two ways of reading:
+//
+//   exact (Shadow::combine == 0): while a pass runs, the value of hot column w is
+//       table[w] + sum of its copies, and a reader sums them all.  No update is delayed, but the
+//       readers of word 0 fetch 17 columns instead of one.  Words 0..7 are hot, with 16, 8, 8, 4,
+//       4, 4, 4, 2 copies (the Zipf shares).
+//   combining (Shadow::combine == 1): readers read the table column only.  What piles up in a
+//       copy is moved into the table by its writers: each copy has a write counter, and the
+//       writer that brings it to a multiple of kFoldEvery swaps the copy to zero (an atomic
+//       exchange, so no concurrent add is lost or counted twice) and adds what it got to the
+//       table column.  A reader misses the updates parked in the copies, fewer than kFoldEvery
+//       per copy.  Words 0..15 are hot, with 32, 16, 16, 8 x 4, 4 x 8, 2 copies.  The launchers
+//       choose this mode only for launches with thousands of work units in flight, where the
+//       parked updates are a small addition to the updates that are invisible anyway because
+//       their work units are still running.
+constexpr int kHotWords = 16;      // hot words of the combining mode; the buffers are sized for it
+constexpr int kShadows = 32;       // copies of word 0 in the combining mode
+constexpr int kHotWordsExact = 8;
+constexpr int kShadowsExact = 16;
+constexpr int kFoldEvery = 8;      // power of two
 
-__device__ __forceinline__ int shadow_copies(int w) {
-  return kShadows >> (31 - __builtin_clz(w + 1));
-}
+constexpr int kCounterStride = 32;  // one write counter per 128-byte line
 
 struct Shadow {
-  float* a;  // [kShadows][kHotWords][d] for table A
-  float* b;  // same for table B
+  float* a;         // [kShadows][kHotWords][d] for table A
+  float* b;         // same for table B
+  unsigned* count;  // [2][kShadows][kHotWords][kCounterStride] write counters (B then A); they
+                    // only ever count up, so they need no clearing between calls
+  int combine;      // 0: exact, 1: combining
 };
+
+__device__ __forceinline__ int shadow_copies(int w, int combine) {
+  const int c = (combine ? kShadows : kShadowsExact) >> (31 - __builtin_clz(w + 1));
+  return c < 2 ? 2 : c;
+}
 
 // ---- where a word's column lives -------------------------------------------------------------
 //
@@ -189,12 +208,20 @@ struct ColRef {
   int flags;   // 0: not resident (skip the word), else kMine or kHead
 };
 
+// The shadow index of `ref` in the mode of `shadow`, or -1.
+__device__ __forceinline__ int hot_index(const ColRef& ref, int combine) {
+  return (combine || ref.hot < kHotWordsExact) ? ref.hot : -1;
+}
+
+// `shadow` is the shadow buffer of ref's table (Shadow::a or Shadow::b).
 template <int R>
 __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const float* shadow,
-                                             int lane, int d) {
+                                             int combine, int lane, int d) {
   load_col<R>(x, ref.col, lane, d);
-  if (ref.hot >= 0) {
-    const int copies = shadow_copies(ref.hot);
+  if (!combine && ref.hot >= 0 && ref.hot < kHotWordsExact) {
+    // two copies per trip: enough loads in flight without inflating the register count of the
+    // callers, which inline this many times
+    const int copies = shadow_copies(ref.hot, 0);
 #pragma unroll 1
     for (int s = 0; s < copies; s += 2) {
       float y0[R], y1[R];
@@ -206,27 +233,61 @@ __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, c
   }
 }
 
-// Column that receives the atomics for `ref` from workgroup number `wg`.
-__device__ __forceinline__ float* scatter_ref(const ColRef& ref, float* shadow, int wg, int d) {
-  if (ref.hot < 0) return ref.col;
-  const int slot = wg & (shadow_copies(ref.hot) - 1);
-  return shadow + ((int64_t)slot * kHotWords + ref.hot) * d;
-}
-
-// A table-relative form of the two helpers above, for kernels that address one pair of tables by
-// word id: column w of `table`, shadowed iff w < kHotWords.
+// Moves what has piled up in a shadow copy into the table column it shadows.
 template <int R>
-__device__ __forceinline__ void load_col_hot(float (&x)[R], const float* table,
-                                             const float* shadow, int w, int lane, int d) {
-  const ColRef ref{const_cast<float*>(table) + (int64_t)w * d, w < kHotWords ? w : -1, kMine};
-  load_col_ref<R>(x, ref, shadow, lane, d);
+__device__ __forceinline__ void fold_copy(float* __restrict__ copy, float* __restrict__ col,
+                                          int lane, int d) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int e = r * kWave + lane;
+    if (r < R - 1 || e < d) {
+      const float v =
+          __hip_atomic_exchange(copy + e, 0.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (v != 0.0f) unsafeAtomicAdd(col + e, v);
+    }
+  }
 }
 
-// Column that receives the atomics for word w from workgroup number `wg`.
-__device__ __forceinline__ float* scatter_target(float* table, float* shadow, int w, int wg,
-                                                 int d) {
-  const ColRef ref{table + (int64_t)w * d, w < kHotWords ? w : -1, kMine};
-  return scatter_ref(ref, shadow, wg, d);
+// col(ref) += x with float atomics.  `shadow` is the shadow buffer of ref's table (sh.a or sh.b),
+// `which` says which table that is (0 = B, 1 = A), `wg` picks the shadow copy.  ref.hot must be
+// wave-uniform.
+template <int R>
+__device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow& sh, int which,
+                                                int wg, const float (&x)[R], int lane, int d) {
+  const int hot = hot_index(ref, sh.combine);
+  if (hot < 0) {
+    atomic_add_col<R>(ref.col, x, lane, d);
+    return;
+  }
+  const int slot = wg & (shadow_copies(hot, sh.combine) - 1);
+  float* const copy = (which ? sh.a : sh.b) + ((int64_t)slot * kHotWords + hot) * d;
+  unsigned seen = 0;
+  if (sh.combine && lane == 0) {
+    unsigned* const counter =
+        sh.count + (((int64_t)which * kShadows + slot) * kHotWords + hot) * kCounterStride;
+    seen = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  atomic_add_col<R>(copy, x, lane, d);
+  if (sh.combine) {
+    const unsigned count = (unsigned)__builtin_amdgcn_readfirstlane((int)seen) + 1u;
+    if ((count & (kFoldEvery - 1)) == 0) fold_copy<R>(copy, ref.col, lane, d);
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void scatter_axpy_ref(const ColRef& ref, const Shadow& sh, int which,
+                                                 int wg, float alpha, const float (&x)[R],
+                                                 int lane, int d) {
+  float y[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) y[r] = alpha * x[r];
+  scatter_add_ref<R>(ref, sh, which, wg, y, lane, d);
+}
+
+// Column w of one table, shadowed iff w < kHotWords (for kernels that address a pair of tables by
+// word id).
+__device__ __forceinline__ ColRef table_ref(float* table, int w, int d) {
+  return ColRef{table + (int64_t)w * d, w < kHotWords ? w : -1, kMine};
 }
 
 // One pair of tables: word w is column w of A / of B; every pair is trained, every column written.

@@ -22,6 +22,8 @@ namespace w2v {
 // max_rows() floats.  The caller of launch_pos / launch_neg provides both buffers zeroed; the
 // launchers leave them zeroed.
 size_t shadow_bytes();
+// Bytes of the write counters of both tables' shadow copies (zero-initialised once, never cleared).
+size_t shadow_counter_bytes();
 
 // Grid size of a persistent kernel: the workgroups that fit on the device at once, but no more
 // than `units / min_units_per_wg` (a workgroup walks at least that many work units, so a small
@@ -31,6 +33,12 @@ hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, in
                            int64_t min_units_per_wg, int64_t* nwg);
 void set_max_workgroups(int n);
 int get_max_workgroups();
+
+// How the hottest columns are updated (w2v_device.h): -1 chosen per launch (the default), 0 exact,
+// 1 combining.  pick_combine gives the mode of a launch of nwg workgroups of waves_per_wg waves.
+void set_hot_update_mode(int mode);
+int get_hot_update_mode();
+int pick_combine(int64_t nwg, int waves_per_wg);
 
 // Adds the shadow copies of the hot columns into A and B and zeroes them.
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);

@@ -17,8 +17,8 @@
 //
 // The update kernel is persistent: a fixed number of workgroups each walk a contiguous range of
 // groups, which bounds the number of groups in flight (and with it the staleness of the Hogwild
-// updates) by the launch size.  The hottest columns are read and updated through their shadow
-// copies (w2v_device.h), so their same-line atomics spread over kShadows lines.
+// updates) by the launch size.  The atomics for the hottest columns go to their shadow copies
+// (w2v_device.h), so their same-line atomics spread over several lines.
 //
 // The reference reads WA/WB without a validity test (:213-214,220-221); here a negative id
 // skips every pair it takes part in, so a bad id cannot become an out-of-bounds access.
@@ -128,7 +128,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       wb[k] = -1;
       if (k < nwb) {
         wb[k] = read_lane(wbl, k);
-        if (wb[k] >= 0) load_col_hot<R>(b[k], B, shadow.b, wb[k], lane, d);
+        if (wb[k] >= 0)
+          load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow.b, shadow.combine, lane, d);
         zero_col<R>(dbb[k]);
       }
     }
@@ -148,7 +149,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
           wa[c] = -1;
           if (j0 + c < jend) {
             wa[c] = read_lane(wal, j0 + c);
-            if (wa[c] >= 0) load_col_hot<R>(a[c], A, shadow.a, wa[c], lane, d);
+            if (wa[c] >= 0)
+              load_col_ref<R>(a[c], table_ref(A, wa[c], d), shadow.a, shadow.combine, lane, d);
           }
         }
         float pre = 0.0f;
@@ -180,7 +182,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
                 axpy<R>(daa, as * g, b[k]);
               }
             }
-            atomic_add_col<R>(scatter_target(A, shadow.a, wa[c], slot, d), daa, lane, d);
+            scatter_add_ref<R>(table_ref(A, wa[c], d), shadow, 1, slot, daa, lane, d);
           }
         }
       }
@@ -189,7 +191,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       if (wb[k] >= 0)
-        atomic_add_col<R>(scatter_target(B, shadow.b, wb[k], slot, d), dbb[k], lane, d);
+        scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d);
     }
   }
 }
@@ -227,6 +229,7 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   if (err != hipSuccess) return err;
   const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
+  shadow.combine = pick_combine(nwg, kNegWaves);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, idlimit,
                      nwa, nwb, groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
   err = hipGetLastError();

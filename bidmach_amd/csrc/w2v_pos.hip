@@ -175,7 +175,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
     const int nc = hi - lo;
 
     // ---- stage: word ids, B columns of every staged position, A columns of the centres.
-    //      Two columns per wave are in flight at a time; hot columns include their shadows.
+    //      Two columns per wave are in flight at a time.
     for (int c0 = wave; c0 < nh; c0 += 2 * kTileWaves) {
       const int c1 = c0 + kTileWaves;
       const int w0 = W[hlo + c0];
@@ -183,8 +183,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const ColRef r0 = tables.b(w0, d);
       const ColRef r1 = tables.b(w1, d);
       float x0[R], x1[R];
-      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.b, lane, d);
-      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.b, lane, d);
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.b, shadow.combine, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.b, shadow.combine, lane, d);
       if (lane == 0) {
         wt[c0] = r0.flags != 0 ? w0 : -1;
         ft[c0] = r0.flags;
@@ -209,8 +209,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const ColRef r0 = tables.a(w0, d);
       const ColRef r1 = tables.a(w1, d);
       float x0[R], x1[R];
-      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.a, lane, d);
-      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.a, lane, d);
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.a, shadow.combine, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.a, shadow.combine, lane, d);
       if (r0.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) a_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
@@ -287,17 +287,17 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
         const ColRef rb = tables.b(wb, d);
         if (rb.flags == 0 || !tables.trained(fi, rb.flags)) continue;
         float b[R];
-        load_col_ref<R>(b, rb, shadow.b, lane, d);
+        load_col_ref<R>(b, rb, shadow.b, shadow.combine, lane, d);
         const float s = wave_sum(dot_partial<R>(a, b));
         const float g = lrate * (1.0f - sat_sigmoid(s));
         axpy<R>(daa, ascale * g, b);
         if (tables.written(rb.flags))
-          atomic_axpy_col<R>(scatter_ref(rb, shadow.b, slot, d), scale_of(wb, vexp, smode) * g, a,
-                             lane, d);
+          scatter_axpy_ref<R>(rb, shadow, 0, slot, scale_of(wb, vexp, smode) * g, a,
+                              lane, d);
         touched = true;
       }
       if (touched && tables.written(fi))
-        atomic_add_col<R>(scatter_ref(tables.a(wi, d), shadow.a, slot, d), daa, lane, d);
+        scatter_add_ref<R>(tables.a(wi, d), shadow, 1, slot, daa, lane, d);
     }
     __syncthreads();
 
@@ -325,8 +325,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
 #pragma unroll
         for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, acol[r * kWave], dbb[r]);
       }
-      atomic_axpy_col<R>(scatter_ref(tables.b(wp, d), shadow.b, slot, d),
-                         scale_of(wp, vexp, smode), dbb, lane, d);
+      scatter_axpy_ref<R>(tables.b(wp, d), shadow, 0, slot,
+                          scale_of(wp, vexp, smode), dbb, lane, d);
     }
     __syncthreads();
   }
@@ -358,6 +358,9 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
 }
 
 size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
+size_t shadow_counter_bytes() {
+  return (size_t)2 * kShadows * kHotWords * kCounterStride * sizeof(unsigned);
+}
 
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d) {
   hipLaunchKernelGGL(fold_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, shadow, d);
@@ -367,6 +370,21 @@ hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, in
 static std::atomic<int> g_max_workgroups{0};
 void set_max_workgroups(int n) { g_max_workgroups.store(n < 0 ? 0 : n); }
 int get_max_workgroups() { return g_max_workgroups.load(); }
+
+static std::atomic<int> g_hot_update_mode{-1};
+void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode == 0 || mode == 1 ? mode : -1); }
+int get_hot_update_mode() { return g_hot_update_mode.load(); }
+
+// The combining mode parks about kFoldEvery/2 updates in each shadow copy, up to ~130 for the
+// most frequent word.  A launch of W waves keeps W work units in flight whose updates are
+// invisible to each other anyway; with the Zipf share of the top word that is several hundred
+// invisible updates of that word per 2048 waves.  Below that size the exact mode is used.
+constexpr int64_t kCombineMinWaves = 2048;
+int pick_combine(int64_t nwg, int waves_per_wg) {
+  const int mode = g_hot_update_mode.load();
+  if (mode == 0 || mode == 1) return mode;
+  return nwg * waves_per_wg >= kCombineMinWaves ? 1 : 0;
+}
 
 hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
                            int64_t min_units_per_wg, int64_t* nwg) {
@@ -488,6 +506,7 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   if (err != hipSuccess) return err;
   const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
   nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  shadow.combine = pick_combine(nwg, kTileWaves);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
                      ntiles, tiles_per_wg, W, LB, UB, tables, lrate, vexp, scale_mode(vexp),
                      shadow);

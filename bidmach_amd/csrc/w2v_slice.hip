@@ -21,8 +21,8 @@
 // and the per-centre positive update used when no tile fits in LDS.  All are wave-per-unit
 // (columns in registers, one column of line-aligned float atomics per written column) and
 // persistent over contiguous ranges of work units, so the work in flight is bounded the same
-// way as in the single-table passes.  The first kHotWords packed columns of part 0 (the most
-// frequent head words) are read and updated through their shadow copies during an update.
+// way as in the single-table passes.  The atomics for the first kHotWords packed columns of part 0
+// (the most frequent head words) go through their shadow copies.
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
@@ -37,13 +37,6 @@ __device__ __forceinline__ float* read_lane_ptr(float* p, int lane) {
 
 __device__ __forceinline__ ColRef read_lane_ref(const ColRef& r, int lane) {
   return ColRef{read_lane_ptr(r.col, lane), read_lane(r.hot, lane), read_lane(r.flags, lane)};
-}
-
-// The forward-only kernels never see non-zero shadows (they are zero between update calls).
-template <bool TRAIN>
-__device__ __forceinline__ ColRef for_pass(ColRef r) {
-  if (!TRAIN) r.hot = -1;
-  return r;
 }
 
 template <int R, int CH, bool TRAIN>
@@ -62,12 +55,12 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
   for (int64_t unit = u_begin + wave; unit < u_end; unit += kWavesPerBlock) {
     const int i = (int)unit;
     const int wi = __builtin_amdgcn_readfirstlane(W[i]);
-    const ColRef pa = for_pass<TRAIN>(tables.a(wi, d));
+    const ColRef pa = tables.a(wi, d);
     if (pa.flags == 0) continue;
     const int jlo = max(LB[i], -i);
     const int jhi = min(UB[i], ncols - 1 - i);
     float a[R];
-    load_col_ref<R>(a, pa, shadow.a, lane, d);
+    load_col_ref<R>(a, pa, shadow.a, TRAIN ? shadow.combine : 1, lane, d);
     float daa[R];
     zero_col<R>(daa);
     const float ascale = TRAIN ? scale_of(wi, vexp, smode) : 1.0f;
@@ -77,7 +70,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
       const int j = base + lane;
       int wl = -1;
       if (j <= jhi && j != 0) wl = W[i + j];
-      const ColRef pb = for_pass<TRAIN>(tables.b(wl, d));
+      const ColRef pb = tables.b(wl, d);
       bool ok = pb.flags != 0;
       if (TRAIN) ok = ok && tables.trained(pa.flags, pb.flags);
       const float sl = (TRAIN && ok) ? scale_of(wl, vexp, smode) : 0.0f;
@@ -103,7 +96,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
         for (int c = 0; c < CH; ++c) {
           if (c < n) {
             rb[c] = read_lane_ref(pb, src[c]);
-            load_col_ref<R>(b[c], rb[c], shadow.b, lane, d);
+            load_col_ref<R>(b[c], rb[c], shadow.b, TRAIN ? shadow.combine : 1, lane, d);
           }
         }
         float pre = 0.0f;
@@ -124,7 +117,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
               const float bs = read_lane(sl, src[c]);
               axpy<R>(daa, ascale * g, b[c]);
               if ((wmask >> src[c]) & 1ull)
-                atomic_axpy_col<R>(scatter_ref(rb[c], shadow.b, slot, d), bs * g, a, lane, d);
+                scatter_axpy_ref<R>(rb[c], shadow, 0, slot, bs * g, a, lane, d);
             }
           }
           touched = true;
@@ -134,7 +127,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
       }
     }
     if (TRAIN && touched && tables.written(pa.flags))
-      atomic_add_col<R>(scatter_ref(pa, shadow.a, slot, d), daa, lane, d);
+      scatter_add_ref<R>(pa, shadow, 1, slot, daa, lane, d);
   }
 
   if (!TRAIN) block_store_partial(wave_sum_f64(lsum), partials);
@@ -157,7 +150,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
   for (int64_t unit = u_begin + wave; unit < u_end; unit += kWavesPerBlock) {
     int wbl = -1;
     if (lane < nwb) wbl = WB[unit * nwb + lane];
-    const ColRef pbl = for_pass<TRAIN>(tables.b(wbl, d));
+    const ColRef pbl = tables.b(wbl, d);
     const float sbl = (TRAIN && pbl.flags != 0) ? scale_of(wbl, vexp, smode) : 0.0f;
 
     float b[MAXB][R];
@@ -171,7 +164,8 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
       if (k < nwb) {
         rb[k] = read_lane_ref(pbl, k);
         fb[k] = rb[k].flags;
-        if (fb[k] != 0) load_col_ref<R>(b[k], rb[k], shadow.b, lane, d);
+        if (fb[k] != 0)
+          load_col_ref<R>(b[k], rb[k], shadow.b, TRAIN ? shadow.combine : 1, lane, d);
         zero_col<R>(dbb[k]);
       }
     }
@@ -179,7 +173,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
       int wal = -1;
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
-      const ColRef pal = for_pass<TRAIN>(tables.a(wal, d));
+      const ColRef pal = tables.a(wal, d);
       const float sal = (TRAIN && pal.flags != 0) ? scale_of(wal, vexp, smode) : 0.0f;
       const int jend = min(nwa - jbase, kWave);
 
@@ -194,7 +188,8 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
           if (j0 + c < jend) {
             ra[c] = read_lane_ref(pal, j0 + c);
             fa[c] = ra[c].flags;
-            if (fa[c] != 0) load_col_ref<R>(a[c], ra[c], shadow.a, lane, d);
+            if (fa[c] != 0)
+              load_col_ref<R>(a[c], ra[c], shadow.a, TRAIN ? shadow.combine : 1, lane, d);
           }
         }
         float pre = 0.0f;
@@ -231,7 +226,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
                 }
               }
               if (tables.written(fa[c]))
-                atomic_add_col<R>(scatter_ref(ra[c], shadow.a, slot, d), daa, lane, d);
+                scatter_add_ref<R>(ra[c], shadow, 1, slot, daa, lane, d);
             }
           }
         } else {
@@ -244,7 +239,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
         if (fb[k] != 0 && tables.written(fb[k]))
-          atomic_add_col<R>(scatter_ref(rb[k], shadow.b, slot, d), dbb[k], lane, d);
+          scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d);
       }
     }
   }
@@ -289,6 +284,7 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ncols, &nwg, &per_wg);
   if (err != hipSuccess) return err;
+  shadow.combine = pick_combine(nwg, kWavesPerBlock);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
                      UB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials, shadow);
   *nparts = nwg;
@@ -304,6 +300,7 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ngroups, &nwg, &per_wg);
   if (err != hipSuccess) return err;
+  shadow.combine = pick_combine(nwg, kWavesPerBlock);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
                      per_wg, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials,
                      shadow);

@@ -59,6 +59,8 @@ SYMBOLS = {
     "w2v_synchronize": (_I, []),
     "w2v_set_max_workgroups": (_I, [_I]),
     "w2v_get_max_workgroups": (_I, []),
+    "w2v_set_hot_update_mode": (_I, [_I]),
+    "w2v_get_hot_update_mode": (_I, []),
     "w2v_max_rows": (_I, []),
     "w2v_max_nwb": (_I, []),
     "w2v_malloc": (_I, [ctypes.POINTER(_P), _SZ]),

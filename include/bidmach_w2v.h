@@ -134,6 +134,18 @@ int w2v_synchronize(void);
 int w2v_set_max_workgroups(int n);
 int w2v_get_max_workgroups(void);
 
+/* How the update operators treat the few most frequent words (ids 0..15), whose columns would
+ * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
+ *   0  exact: their atomics are spread over shadow copies and every reader sums the copies, so no
+ *      update is ever delayed;
+ *   1  combining: readers read the table only and the copies are moved into the table every few
+ *      writes, which hides up to about a hundred updates of the most frequent word from readers
+ *      for a few microseconds and is about 20 % faster on a raw Zipf stream;
+ *  -1  (default) combining for launches with at least 2048 wavefronts in flight, where that many
+ *      updates are invisible to each other anyway, exact for smaller ones. */
+int w2v_set_hot_update_mode(int mode);
+int w2v_get_hot_update_mode(void);
+
 /* Limits of the kernels: largest nrows and largest nwb. */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
