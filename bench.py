@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # --pmc WRITE_SIZE on this same command (summaries under profiles/), scaled by what the same
 # counters read for a plain copy of known size in the same run (FETCH x2.0, WRITE x1.0).
 MEASURED_TRAFFIC_BYTES = {
-    "sgns_v1m_d300_w5_neg5_fp32": {"neg_kernel": 33.84e9, "pos_kernel": 5.98e9},
+    "sgns_v1m_d300_w5_neg5_fp32": {"neg_kernel": 29.35e9, "pos_kernel": 4.88e9},
 }
 
 WORKLOADS = {
@@ -124,6 +124,9 @@ def main():
     ap.add_argument("--wsample", type=float, default=0.0,
                     help="frequent-word subsampling threshold of the reference caller (its default "
                          "is 1e-4); 0 = the raw stream the headline metric is defined on")
+    ap.add_argument("--hot-mode", type=int, default=-1, choices=[-1, 0, 1],
+                    help="w2v_set_hot_update_mode: -1 the library's per-launch choice (default), "
+                         "0 exact shadow copies, 1 combining shadow copies")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -141,6 +144,8 @@ def main():
     from bidmach_amd.cumach import CUMACH, Timer, check, synchronize
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    from bidmach_amd.cumach import load_library
+    load_library().w2v_set_hot_update_mode(args.hot_mode)
     cfg = WORKLOADS[args.workload]
     d, V, n = cfg["dim"], cfg["vocab"], cfg["tokens"]
     K, Wm = args.steps, args.warmup
@@ -293,6 +298,8 @@ def main():
     if evaluating:
         out["config"]["mode"] = "eval"
         out["roofline"]["traffic"] = None
+    if args.hot_mode != -1:
+        out["config"]["hot_update_mode"] = args.hot_mode
     if args.wsample > 0.0:
         out["config"]["wsample"] = args.wsample
         out["roofline"]["traffic"] = None

@@ -77,6 +77,9 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   out->a = ts.shadow[dev];
   out->b = ts.shadow[dev] + bytes / sizeof(float);
   out->count = reinterpret_cast<unsigned*>(ts.shadow[dev] + 2 * (bytes / sizeof(float)));
+  out->hot_seen = reinterpret_cast<int*>(out->count + (size_t)2 * w2v::kShadows * w2v::kHotWords *
+                                                          w2v::kCounterStride);
+  out->hot_total = 0;
   out->combine = 0;
   return hipSuccess;
 }

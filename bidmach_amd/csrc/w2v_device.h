@@ -157,8 +157,11 @@ __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float a
 // columns the critical path of the whole pass.  The atomics for a hot column therefore go to one
 // of several shadow copies of it (chosen by the workgroup index) in a scratch buffer that is zero
 // between calls, so the same-line queue is spread over several lines.  A small kernel moves what
-// is left in the copies into the table at the end of the call.  Two ways of reading:
+// is left in the copies into the table at the end of the call.  Three modes (HotMode):
 //
+//   off: no shadow copies; every column is read and updated in place.  Chosen inside the kernel
+//       when the launch holds few hot words (fewer than 1/kHotShareDen of its ids, counted by a
+//       small kernel beforehand), as after frequent-word subsampling.
 //   exact (Shadow::combine == 0): while a pass runs, the value of hot column w is
 //       table[w] + sum of its copies, and a reader sums them all.  No update is delayed, but the
 //       readers of word 0 fetch 17 columns instead of one.  Words 0..7 are hot, with 16, 8, 8, 4,
@@ -172,24 +175,40 @@ __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float a
 //       choose this mode only for launches with thousands of work units in flight, where the
 //       parked updates are a small addition to the updates that are invisible anyway because
 //       their work units are still running.
-constexpr int kHotWords = 16;      // hot words of the combining mode; the buffers are sized for it
-constexpr int kShadows = 32;       // copies of word 0 in the combining mode
+constexpr int kHotWords = 16;  // hot words of the combining mode; the buffers are sized for it
+constexpr int kShadows = 32;   // copies of word 0 in the combining mode
 constexpr int kHotWordsExact = 8;
 constexpr int kShadowsExact = 16;
-constexpr int kFoldEvery = 8;      // power of two
+constexpr int kFoldEvery = 8;  // power of two; 16 is 6 % faster and parks twice as many updates
 
 constexpr int kCounterStride = 32;  // one write counter per 128-byte line
+
+enum HotMode : int { kHotExact = 0, kHotCombining = 1, kHotOff = 2 };
+constexpr int kHotShareDen = 16;  // shadows are used if >= 1/16 of a launch's ids are hot words
 
 struct Shadow {
   float* a;         // [kShadows][kHotWords][d] for table A
   float* b;         // same for table B
   unsigned* count;  // [2][kShadows][kHotWords][kCounterStride] write counters (B then A); they
                     // only ever count up, so they need no clearing between calls
-  int combine;      // 0: exact, 1: combining
+  int* hot_seen;        // how many of the launch's `hot_total` word ids are below kHotWords,
+  long long hot_total;  // counted on the device before the launch; hot_total == 0: not counted
+  int combine;          // kHotExact or kHotCombining (kHotOff once resolved in a kernel)
 };
 
+// The mode a kernel runs in: the launcher's, unless the ids of this launch hold too few hot words
+// for shadow copies to pay (subsampled or re-numbered vocabularies), in which case every column is
+// read and updated in place.
+__device__ __forceinline__ Shadow resolve_hot_mode(Shadow sh) {
+  if (sh.hot_total > 0) {
+    const long long seen = __builtin_amdgcn_readfirstlane(*sh.hot_seen);
+    if (seen * kHotShareDen < sh.hot_total) sh.combine = kHotOff;
+  }
+  return sh;
+}
+
 __device__ __forceinline__ int shadow_copies(int w, int combine) {
-  const int c = (combine ? kShadows : kShadowsExact) >> (31 - __builtin_clz(w + 1));
+  const int c = (combine == kHotCombining ? kShadows : kShadowsExact) >> (31 - __builtin_clz(w + 1));
   return c < 2 ? 2 : c;
 }
 
@@ -210,7 +229,8 @@ struct ColRef {
 
 // The shadow index of `ref` in the mode of `shadow`, or -1.
 __device__ __forceinline__ int hot_index(const ColRef& ref, int combine) {
-  return (combine || ref.hot < kHotWordsExact) ? ref.hot : -1;
+  if (combine == kHotOff) return -1;
+  return (combine == kHotCombining || ref.hot < kHotWordsExact) ? ref.hot : -1;
 }
 
 // `shadow` is the shadow buffer of ref's table (Shadow::a or Shadow::b).
@@ -218,7 +238,7 @@ template <int R>
 __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const float* shadow,
                                              int combine, int lane, int d) {
   load_col<R>(x, ref.col, lane, d);
-  if (!combine && ref.hot >= 0 && ref.hot < kHotWordsExact) {
+  if (combine == kHotExact && ref.hot >= 0 && ref.hot < kHotWordsExact) {
     // two copies per trip: enough loads in flight without inflating the register count of the
     // callers, which inline this many times
     const int copies = shadow_copies(ref.hot, 0);
@@ -262,13 +282,13 @@ __device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow&
   const int slot = wg & (shadow_copies(hot, sh.combine) - 1);
   float* const copy = (which ? sh.a : sh.b) + ((int64_t)slot * kHotWords + hot) * d;
   unsigned seen = 0;
-  if (sh.combine && lane == 0) {
+  if (sh.combine == kHotCombining && lane == 0) {
     unsigned* const counter =
         sh.count + (((int64_t)which * kShadows + slot) * kHotWords + hot) * kCounterStride;
     seen = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   atomic_add_col<R>(copy, x, lane, d);
-  if (sh.combine) {
+  if (sh.combine == kHotCombining) {
     const unsigned count = (unsigned)__builtin_amdgcn_readfirstlane((int)seen) + 1u;
     if ((count & (kFoldEvery - 1)) == 0) fold_copy<R>(copy, ref.col, lane, d);
   }

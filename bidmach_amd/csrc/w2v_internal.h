@@ -22,7 +22,8 @@ namespace w2v {
 // max_rows() floats.  The caller of launch_pos / launch_neg provides both buffers zeroed; the
 // launchers leave them zeroed.
 size_t shadow_bytes();
-// Bytes of the write counters of both tables' shadow copies (zero-initialised once, never cleared).
+// Bytes of the write counters of both tables' shadow copies plus the hot-word count of a launch
+// (zero-initialised once; the counters are never cleared, the count is cleared by launch_fold).
 size_t shadow_counter_bytes();
 
 // Grid size of a persistent kernel: the workgroups that fit on the device at once, but no more
@@ -35,10 +36,13 @@ void set_max_workgroups(int n);
 int get_max_workgroups();
 
 // How the hottest columns are updated (w2v_device.h): -1 chosen per launch (the default), 0 exact,
-// 1 combining.  pick_combine gives the mode of a launch of nwg workgroups of waves_per_wg waves.
+// 1 combining.  prepare_hot_mode fills in the mode fields of `shadow` for a launch of nwg workgroups
+// of waves_per_wg waves over the n word ids `ids` (device memory); in the default mode it first
+// enqueues the count of hot words among them.
 void set_hot_update_mode(int mode);
 int get_hot_update_mode();
-int pick_combine(int64_t nwg, int waves_per_wg);
+hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64_t nwg,
+                            int waves_per_wg, Shadow* shadow);
 
 // Adds the shadow copies of the hot columns into A and B and zeroes them.
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);

@@ -104,8 +104,9 @@ template <int R, int MAXB, int CHA>
 __global__ void __launch_bounds__(kNegThreads, W2V_NEG_WAVES_PER_EU)
 neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t groups_per_wg,
                  const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
-                 float lrate, float vexp, int smode, Shadow shadow) {
+                 float lrate, float vexp, int smode, Shadow shadow_arg) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
+  const Shadow shadow = resolve_hot_mode(shadow_arg);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
@@ -229,7 +230,8 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   if (err != hipSuccess) return err;
   const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
-  shadow.combine = pick_combine(nwg, kNegWaves);
+  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nwg, kNegWaves, &shadow);
+  if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, idlimit,
                      nwa, nwb, groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
   err = hipGetLastError();

@@ -150,8 +150,9 @@ __global__ void __launch_bounds__(kTileThreads)
 pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg,
                 const int* __restrict__ W, const int* __restrict__ LB,
                 const int* __restrict__ UB, Tables tables, float lrate, float vexp, int smode,
-                Shadow shadow) {
+                Shadow shadow_arg) {
   extern __shared__ float lds[];
+  const Shadow shadow = resolve_hot_mode(shadow_arg);
   constexpr int dp = R * kWave;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -355,11 +356,34 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
     }
     if (any) table[(int64_t)w * d + e] += sum;
   }
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *shadow.hot_seen = 0;
+}
+
+// Counts the word ids below kHotWords into *out (zero before the launch): one atomic per block,
+// so the adds to the one counter do not queue up.
+__global__ void __launch_bounds__(kBlock)
+count_hot_kernel(const int* __restrict__ ids, int64_t n, int* out) {
+  __shared__ int s_part[kWavesPerBlock];
+  int local = 0;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int w = ids[i];
+    local += (w >= 0 && w < kHotWords) ? 1 : 0;
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) local += __shfl_xor(local, m, kWave);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
+    if (total != 0) atomicAdd(out, total);
+  }
 }
 
 size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
 size_t shadow_counter_bytes() {
-  return (size_t)2 * kShadows * kHotWords * kCounterStride * sizeof(unsigned);
+  return ((size_t)2 * kShadows * kHotWords + 1) * kCounterStride * sizeof(unsigned);
 }
 
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d) {
@@ -375,15 +399,30 @@ static std::atomic<int> g_hot_update_mode{-1};
 void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode == 0 || mode == 1 ? mode : -1); }
 int get_hot_update_mode() { return g_hot_update_mode.load(); }
 
-// The combining mode parks about kFoldEvery/2 updates in each shadow copy, up to ~130 for the
-// most frequent word.  A launch of W waves keeps W work units in flight whose updates are
+// Chooses how a launch of nwg workgroups treats the hot words (Shadow::combine and the hot-word
+// count the kernels consult).  The combining mode parks up to kFoldEvery - 1 updates in each shadow
+// copy, a couple of hundred for the most frequent word.  A launch of W waves keeps W work units in flight whose updates are
 // invisible to each other anyway; with the Zipf share of the top word that is several hundred
 // invisible updates of that word per 2048 waves.  Below that size the exact mode is used.
 constexpr int64_t kCombineMinWaves = 2048;
-int pick_combine(int64_t nwg, int waves_per_wg) {
+hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64_t nwg,
+                            int waves_per_wg, Shadow* shadow) {
   const int mode = g_hot_update_mode.load();
-  if (mode == 0 || mode == 1) return mode;
-  return nwg * waves_per_wg >= kCombineMinWaves ? 1 : 0;
+  shadow->hot_total = 0;
+  if (mode == kHotExact || mode == kHotCombining) {
+    shadow->combine = mode;
+    return hipSuccess;
+  }
+  shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
+  if (n <= 0) return hipSuccess;
+  // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
+  // read the count from memory, the host does not wait for it).
+  const int64_t want = (n + 16 * kBlock - 1) / (16 * kBlock);
+  const unsigned grid = (unsigned)(want < 1 ? 1 : (want > 256 ? 256 : want));
+  hipLaunchKernelGGL(count_hot_kernel, dim3(grid), dim3(kBlock), 0, stream, ids, n,
+                     shadow->hot_seen);
+  shadow->hot_total = n;
+  return hipGetLastError();
 }
 
 hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
@@ -506,7 +545,8 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   if (err != hipSuccess) return err;
   const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
   nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
-  shadow.combine = pick_combine(nwg, kTileWaves);
+  err = prepare_hot_mode(stream, W, ncols, nwg, kTileWaves, &shadow);
+  if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
                      ntiles, tiles_per_wg, W, LB, UB, tables, lrate, vexp, scale_mode(vexp),
                      shadow);

@@ -44,7 +44,8 @@ __global__ void __launch_bounds__(kBlock)
 slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ W,
                  const int* __restrict__ LB, const int* __restrict__ UB, SlicedTables tables,
                  float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
-                 Shadow shadow) {
+                 Shadow shadow_arg) {
+  const Shadow shadow = TRAIN ? resolve_hot_mode(shadow_arg) : shadow_arg;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;
@@ -60,7 +61,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
     const int jlo = max(LB[i], -i);
     const int jhi = min(UB[i], ncols - 1 - i);
     float a[R];
-    load_col_ref<R>(a, pa, shadow.a, TRAIN ? shadow.combine : 1, lane, d);
+    load_col_ref<R>(a, pa, shadow.a, TRAIN ? shadow.combine : kHotOff, lane, d);
     float daa[R];
     zero_col<R>(daa);
     const float ascale = TRAIN ? scale_of(wi, vexp, smode) : 1.0f;
@@ -96,7 +97,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
         for (int c = 0; c < CH; ++c) {
           if (c < n) {
             rb[c] = read_lane_ref(pb, src[c]);
-            load_col_ref<R>(b[c], rb[c], shadow.b, TRAIN ? shadow.combine : 1, lane, d);
+            load_col_ref<R>(b[c], rb[c], shadow.b, TRAIN ? shadow.combine : kHotOff, lane, d);
           }
         }
         float pre = 0.0f;
@@ -138,8 +139,9 @@ __global__ void __launch_bounds__(kBlock, 3)
 slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
                  const int* __restrict__ WA, const int* __restrict__ WB, SlicedTables tables,
                  float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
-                 Shadow shadow) {
+                 Shadow shadow_arg) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
+  const Shadow shadow = TRAIN ? resolve_hot_mode(shadow_arg) : shadow_arg;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;
@@ -165,7 +167,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
         rb[k] = read_lane_ref(pbl, k);
         fb[k] = rb[k].flags;
         if (fb[k] != 0)
-          load_col_ref<R>(b[k], rb[k], shadow.b, TRAIN ? shadow.combine : 1, lane, d);
+          load_col_ref<R>(b[k], rb[k], shadow.b, TRAIN ? shadow.combine : kHotOff, lane, d);
         zero_col<R>(dbb[k]);
       }
     }
@@ -189,7 +191,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
             ra[c] = read_lane_ref(pal, j0 + c);
             fa[c] = ra[c].flags;
             if (fa[c] != 0)
-              load_col_ref<R>(a[c], ra[c], shadow.a, TRAIN ? shadow.combine : 1, lane, d);
+              load_col_ref<R>(a[c], ra[c], shadow.a, TRAIN ? shadow.combine : kHotOff, lane, d);
           }
         }
         float pre = 0.0f;
@@ -284,7 +286,10 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ncols, &nwg, &per_wg);
   if (err != hipSuccess) return err;
-  shadow.combine = pick_combine(nwg, kWavesPerBlock);
+  if (TRAIN) {
+    err = prepare_hot_mode(stream, W, ncols, nwg, kWavesPerBlock, &shadow);
+    if (err != hipSuccess) return err;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
                      UB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials, shadow);
   *nparts = nwg;
@@ -300,7 +305,10 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
   int64_t nwg = 0, per_wg = 0;
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ngroups, &nwg, &per_wg);
   if (err != hipSuccess) return err;
-  shadow.combine = pick_combine(nwg, kWavesPerBlock);
+  if (TRAIN) {
+    err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nwg, kWavesPerBlock, &shadow);
+    if (err != hipSuccess) return err;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
                      per_wg, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials,
                      shadow);

@@ -136,13 +136,15 @@ int w2v_get_max_workgroups(void);
 
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
  * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
- *   0  exact: their atomics are spread over shadow copies and every reader sums the copies, so no
- *      update is ever delayed;
- *   1  combining: readers read the table only and the copies are moved into the table every few
- *      writes, which hides up to about a hundred updates of the most frequent word from readers
- *      for a few microseconds and is about 20 % faster on a raw Zipf stream;
- *  -1  (default) combining for launches with at least 2048 wavefronts in flight, where that many
- *      updates are invisible to each other anyway, exact for smaller ones. */
+ *   0  exact: their atomics are spread over shadow copies and every reader sums the copies;
+ *   1  combining: readers read the table only and a copy is moved into the table on every 8th
+ *      write to it, which hides fewer than 8 updates per copy (a couple of hundred of the most
+ *      frequent word) from readers for a few microseconds; about 20 % faster than 0 on a raw
+ *      Zipf stream;
+ *  -1  (default) decided per launch on the device: no shadow copies at all unless at least 1/16
+ *      of the launch's word ids are among those 16 (they are not after frequent-word subsampling);
+ *      otherwise combining for launches with at least 2048 wavefronts in flight, where that many
+ *      updates are invisible to each other anyway, and exact for smaller ones. */
 int w2v_set_hot_update_mode(int mode);
 int w2v_get_hot_update_mode(void);
 
