@@ -8,7 +8,11 @@
 //   - gather followed by atomic scatter,
 //   - a plain load-add-store of the same columns (no atomics),
 // for ids drawn uniformly, from Zipf(1.0), and from the mix a negative pass sees (5 ids from
-// unigram^0.75 + 5 from Zipf(1.0)), the latter also with shadow copies of the 8 hottest columns.
+// unigram^0.75 + 5 from Zipf(1.0)); the latter also with the ids below 8 (below 1024) replaced by
+// uniform ones (what a perfect spreading of the hot columns would give), with shadow copies of the
+// 8 hottest columns that every reader sums ("exact"), and with shadow copies of the 16 hottest
+// columns that writers fold into the table every 8th write while readers read the table only
+// ("combining").
 // Also a plain 1.2 GB copy as the streaming reference.  The library's design decisions (few,
 // line-aligned atomics; LDS tiles; shadow copies) follow from these numbers.
 //
@@ -102,6 +106,100 @@ touch(const int* __restrict__ ids, int nunits, float* T, float* S, float* sink) 
   if (MODE == kGather && acc == 123.456f) sink[0] = acc;
 }
 
+constexpr int CHOT = 16, CSHADOWS = 32, FOLD_EVERY = 8, CSTRIDE = 32;
+
+__device__ __forceinline__ int copies_of(int w) {
+  const int c = CSHADOWS >> (31 - __builtin_clz(w + 1));
+  return c < 2 ? 2 : c;
+}
+
+// Gather + line-aligned atomics; the atomics for ids below CHOT go to a shadow copy, and the writer
+// that brings the copy's counter to a multiple of FOLD_EVERY swaps the copy out and adds it to the
+// table column.  Persistent: workgroup b walks units [b*per_wg, (b+1)*per_wg).
+__global__ void __launch_bounds__(256)
+touch_combining(const int* __restrict__ ids, int nunits, long per_wg, float* T, float* S,
+                unsigned* C) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long ubeg = (long)blockIdx.x * per_wg;
+  const long uend = ubeg + per_wg < nunits ? ubeg + per_wg : nunits;
+  for (long unit = ubeg + wave; unit < uend; unit += 4) {
+    const int mine = lane < K ? ids[unit * K + lane] : 0;
+    // lane k takes the ticket of column k's write now, so it is back when the write happens
+    unsigned ticket = 0;
+    if (lane < K && mine < CHOT) {
+      const int slot = blockIdx.x & (copies_of(mine) - 1);
+      ticket = __hip_atomic_fetch_add(C + ((long)slot * CHOT + mine) * CSTRIDE, 1u,
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float x[K][R];
+    int id[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      id[k] = __builtin_amdgcn_readlane(mine, k);
+      const float* col = T + (long)id[k] * D;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int e = r * 64 + lane;
+        x[k][r] = e < D ? col[e] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      float* const tab = T + (long)id[k] * D;
+      float* col = tab;
+      const bool hot = id[k] < CHOT;
+      if (hot) col = S + ((long)(blockIdx.x & (copies_of(id[k]) - 1)) * CHOT + id[k]) * D;
+      const int mis = (int)((reinterpret_cast<uintptr_t>(col) >> 2) & 31u);
+#pragma unroll
+      for (int r = 0; r <= R; ++r) {
+        const int e = r * 64 + lane - mis;
+        if (e >= 0 && e < D) unsafeAtomicAdd(col + e, x[k][r < R ? r : 0] * 1e-9f);
+      }
+      if (hot) {
+        const unsigned count = (unsigned)__builtin_amdgcn_readlane((int)ticket, k) + 1u;
+        if ((count & (FOLD_EVERY - 1)) == 0) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            const int e = r * 64 + lane;
+            if (e < D) {
+              const float v = __hip_atomic_exchange(col + e, 0.0f, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+              if (v != 0.0f) unsafeAtomicAdd(tab + e, v);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+static float run_combining(const int* ids, int nunits, float* T) {
+  float* S;
+  unsigned* C;
+  CK(hipMalloc(&S, (size_t)CSHADOWS * CHOT * D * 4));
+  CK(hipMemset(S, 0, (size_t)CSHADOWS * CHOT * D * 4));
+  CK(hipMalloc(&C, (size_t)CSHADOWS * CHOT * CSTRIDE * 4));
+  CK(hipMemset(C, 0, (size_t)CSHADOWS * CHOT * CSTRIDE * 4));
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  const int nwg = 768;
+  const long per_wg = ((long)nunits + nwg - 1) / nwg;
+  hipLaunchKernelGGL(touch_combining, dim3(nwg), dim3(256), 0, 0, ids, nunits, per_wg, T, S, C);
+  CK(hipDeviceSynchronize());
+  CK(hipEventRecord(e0));
+  for (int i = 0; i < 3; ++i)
+    hipLaunchKernelGGL(touch_combining, dim3(nwg), dim3(256), 0, 0, ids, nunits, per_wg, T, S, C);
+  CK(hipEventRecord(e1));
+  CK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  CK(hipFree(S));
+  CK(hipFree(C));
+  return ms / 3;
+}
+
 __global__ void copy_kernel(const float4* __restrict__ a, float4* __restrict__ b, long n) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long stride = (long)gridDim.x * blockDim.x;
@@ -177,8 +275,20 @@ int main() {
            names[k], g, gb / g * 1e3, a, gb / a * 1e3, al, gb / al * 1e3, ga, ls);
     if (k == 2) {
       const float sh = run<kShadowed>(d_ids, NU, T, S, sink);
-      printf("%-34s gather + aligned atomics with %d shadow copies of the %d hottest columns "
-             "%6.2f ms\n", names[k], SHADOWS, HOT, sh);
+      printf("%-34s gather + aligned atomics, exact shadows (%d copies of the %d hottest columns, "
+             "readers sum them) %6.2f ms\n", names[k], SHADOWS, HOT, sh);
+      const float cb = run_combining(d_ids, NU, T);
+      printf("%-34s gather + aligned atomics, combining shadows (%d hottest columns, folded "
+             "every %d writes, readers read the table) %6.2f ms\n", names[k], CHOT, FOLD_EVERY, cb);
+      for (int H : {8, 1024}) {
+        std::vector<int> spread(ids[2]);
+        for (auto& v : spread)
+          if (v < H) v = (int)(U(rng) * V) % V;
+        CK(hipMemcpy(d_ids, spread.data(), n * 4, hipMemcpyHostToDevice));
+        const float ga2 = run<kGatherAtomicAligned>(d_ids, NU, T, S, sink);
+        printf("%-34s gather + aligned atomics with the ids below %d made uniform %6.2f ms\n",
+               names[k], H, ga2);
+      }
     }
     fflush(stdout);
   }

@@ -268,12 +268,29 @@ __device__ __forceinline__ void fold_copy(float* __restrict__ copy, float* __res
   }
 }
 
-// col(ref) += x with float atomics.  `shadow` is the shadow buffer of ref's table (sh.a or sh.b),
-// `which` says which table that is (0 = B, 1 = A), `wg` picks the shadow copy.  ref.hot must be
-// wave-uniform.
+// Announces a write to the column with shadow index `hot` (ColRef::hot; -1 for none) and returns
+// the value of its copy's write counter before this write.  Lanes may ask for different columns.
+// The returning atomic takes a few microseconds, so callers take the ticket well before the write
+// it belongs to.  0 when the write will not go to a combining shadow copy.
+__device__ __forceinline__ unsigned hot_ticket(const Shadow& sh, int which, int wg, int hot) {
+  if (sh.combine != kHotCombining || hot < 0) return 0u;
+  const int slot = wg & (shadow_copies(hot, kHotCombining) - 1);
+  unsigned* const counter =
+      sh.count + (((int64_t)which * kShadows + slot) * kHotWords + hot) * kCounterStride;
+  return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ unsigned read_lane(unsigned x, int lane) {
+  return (unsigned)__builtin_amdgcn_readlane((int)x, lane);
+}
+
+// col(ref) += x with float atomics.  `which` says which table ref belongs to (0 = B, 1 = A), `wg`
+// picks the shadow copy, `ticket` is the wave-uniform result of hot_ticket for this write.
+// ref.hot must be wave-uniform.
 template <int R>
 __device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow& sh, int which,
-                                                int wg, const float (&x)[R], int lane, int d) {
+                                                int wg, const float (&x)[R], int lane, int d,
+                                                unsigned ticket) {
   const int hot = hot_index(ref, sh.combine);
   if (hot < 0) {
     atomic_add_col<R>(ref.col, x, lane, d);
@@ -281,17 +298,28 @@ __device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow&
   }
   const int slot = wg & (shadow_copies(hot, sh.combine) - 1);
   float* const copy = (which ? sh.a : sh.b) + ((int64_t)slot * kHotWords + hot) * d;
-  unsigned seen = 0;
-  if (sh.combine == kHotCombining && lane == 0) {
-    unsigned* const counter =
-        sh.count + (((int64_t)which * kShadows + slot) * kHotWords + hot) * kCounterStride;
-    seen = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
   atomic_add_col<R>(copy, x, lane, d);
-  if (sh.combine == kHotCombining) {
-    const unsigned count = (unsigned)__builtin_amdgcn_readfirstlane((int)seen) + 1u;
-    if ((count & (kFoldEvery - 1)) == 0) fold_copy<R>(copy, ref.col, lane, d);
-  }
+  if (sh.combine == kHotCombining && ((ticket + 1u) & (kFoldEvery - 1)) == 0)
+    fold_copy<R>(copy, ref.col, lane, d);
+}
+
+// The same for callers on a rarely taken path: takes the ticket on the spot.
+template <int R>
+__device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow& sh, int which,
+                                                int wg, const float (&x)[R], int lane, int d) {
+  const unsigned mine = lane == 0 ? hot_ticket(sh, which, wg, ref.hot) : 0u;
+  const unsigned ticket = (unsigned)__builtin_amdgcn_readfirstlane((int)mine);
+  scatter_add_ref<R>(ref, sh, which, wg, x, lane, d, ticket);
+}
+
+template <int R>
+__device__ __forceinline__ void scatter_axpy_ref(const ColRef& ref, const Shadow& sh, int which,
+                                                 int wg, float alpha, const float (&x)[R],
+                                                 int lane, int d, unsigned ticket) {
+  float y[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) y[r] = alpha * x[r];
+  scatter_add_ref<R>(ref, sh, which, wg, y, lane, d, ticket);
 }
 
 template <int R>

@@ -120,6 +120,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
     if (lane < nwb) wbl = WB[unit * nwb + lane];
     if (wbl >= idlimit) wbl = -1;  // word2vecNegFilt: ids beyond the resident columns are skipped
     const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
+    // tickets for the writes to hot B columns at the end of the group, taken now
+    const unsigned tkb = hot_ticket(shadow, 0, slot, (wbl >= 0 && wbl < kHotWords) ? wbl : -1);
 
     float b[MAXB][R];
     float dbb[MAXB][R];
@@ -140,6 +142,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
       if (wal >= idlimit) wal = -1;
       const float sal = wal >= 0 ? scale_of(wal, vexp, smode) : 0.0f;
+      const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
       const int jend = min(nwa - jbase, kWave);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -183,7 +186,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
                 axpy<R>(daa, as * g, b[k]);
               }
             }
-            scatter_add_ref<R>(table_ref(A, wa[c], d), shadow, 1, slot, daa, lane, d);
+            scatter_add_ref<R>(table_ref(A, wa[c], d), shadow, 1, slot, daa, lane, d,
+                               read_lane(tka, j0 + c));
           }
         }
       }
@@ -192,7 +196,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       if (wb[k] >= 0)
-        scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d);
+        scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d,
+                           read_lane(tkb, k));
     }
   }
 }

@@ -145,8 +145,10 @@ __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
 
 // `tables` is PlainTables (word2vecPos) or SlicedTables (word2vecPosSlice): it places a word's
 // column and says which pairs are trained and which columns are written.
+// Up to R = 7 two workgroups fit in a CU's LDS, which needs four waves per SIMD: the register
+// budget is held to that.
 template <int R, class Tables>
-__global__ void __launch_bounds__(kTileThreads)
+__global__ void __launch_bounds__(kTileThreads, (R <= 7 ? 4 : 2))
 pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg,
                 const int* __restrict__ W, const int* __restrict__ LB,
                 const int* __restrict__ UB, Tables tables, float lrate, float vexp, int smode,
@@ -230,6 +232,9 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const int wi = wt[i - hlo];
       if (wi < 0) continue;
       const int fi = Tables::kSliced ? ft[i - hlo] : kMine;
+      // ticket for the write to this centre's A column at the end of the iteration, taken now
+      const ColRef ra = tables.a(wi, d);
+      const unsigned tka = lane == 0 ? hot_ticket(shadow, 1, slot, ra.hot) : 0u;
       const int jlo = max(LB[i], -i);
       const int jhi = min(UB[i], ncols - 1 - i);
       float a[R];
@@ -298,7 +303,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
         touched = true;
       }
       if (touched && tables.written(fi))
-        scatter_add_ref<R>(tables.a(wi, d), shadow, 1, slot, daa, lane, d);
+        scatter_add_ref<R>(ra, shadow, 1, slot, daa, lane, d,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)tka));
     }
     __syncthreads();
 
@@ -316,6 +322,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       if (lane < gw && i >= lo && i < hi && i != p) gl = G[(i - lo) * gw + (p - i + Sh)];
       unsigned long long mask = __ballot(gl != 0.0f);
       if (mask == 0ull) continue;
+      const ColRef rp = tables.b(wp, d);
+      const unsigned tkb = lane == 0 ? hot_ticket(shadow, 0, slot, rp.hot) : 0u;
       float dbb[R];
       zero_col<R>(dbb);
       while (mask != 0ull) {
@@ -326,8 +334,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
 #pragma unroll
         for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, acol[r * kWave], dbb[r]);
       }
-      scatter_axpy_ref<R>(tables.b(wp, d), shadow, 0, slot,
-                          scale_of(wp, vexp, smode), dbb, lane, d);
+      scatter_axpy_ref<R>(rp, shadow, 0, slot, scale_of(wp, vexp, smode), dbb, lane, d,
+                          (unsigned)__builtin_amdgcn_readfirstlane((int)tkb));
     }
     __syncthreads();
   }

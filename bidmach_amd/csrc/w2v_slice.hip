@@ -154,6 +154,9 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     if (lane < nwb) wbl = WB[unit * nwb + lane];
     const ColRef pbl = tables.b(wbl, d);
     const float sbl = (TRAIN && pbl.flags != 0) ? scale_of(wbl, vexp, smode) : 0.0f;
+    // tickets for the writes to hot B columns at the end of the group, taken now
+    const unsigned tkb =
+        (TRAIN && tables.written(pbl.flags)) ? hot_ticket(shadow, 0, slot, pbl.hot) : 0u;
 
     float b[MAXB][R];
     float dbb[MAXB][R];
@@ -177,6 +180,8 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
       const ColRef pal = tables.a(wal, d);
       const float sal = (TRAIN && pal.flags != 0) ? scale_of(wal, vexp, smode) : 0.0f;
+      const unsigned tka =
+          (TRAIN && tables.written(pal.flags)) ? hot_ticket(shadow, 1, slot, pal.hot) : 0u;
       const int jend = min(nwa - jbase, kWave);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -228,7 +233,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
                 }
               }
               if (tables.written(fa[c]))
-                scatter_add_ref<R>(ra[c], shadow, 1, slot, daa, lane, d);
+                scatter_add_ref<R>(ra[c], shadow, 1, slot, daa, lane, d, read_lane(tka, j0 + c));
             }
           }
         } else {
@@ -241,7 +246,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
         if (fb[k] != 0 && tables.written(fb[k]))
-          scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d);
+          scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d, read_lane(tkb, k));
       }
     }
   }
