@@ -129,7 +129,8 @@ def lz4_stream_write(f, payload, block_size=LZ4_BLOCK):
 
 
 def lz4_stream_read(f, verify=True):
-    """Reads an lz4-java block stream to its end marker (or end of file); returns the bytes."""
+    """Reads an lz4-java block stream to its end marker (or end of file); returns the bytes as a
+    writable buffer."""
     out = io.BytesIO()
     while True:
         head = f.read(21)
@@ -159,7 +160,7 @@ def lz4_stream_read(f, verify=True):
         if verify and _checksum(chunk) != check:
             raise MatFileError("LZ4Block checksum mismatch")
         out.write(chunk)
-    return out.getvalue()
+    return out.getbuffer()
 
 
 def _encode(m):
@@ -212,16 +213,16 @@ def saveMat(path, m):
 
 
 def loadMat(path):
-    """Reads a dense matrix file; returns a Fortran-ordered (nrows, ncols) array."""
+    """Reads a dense matrix file; returns a writable, Fortran-ordered (nrows, ncols) array."""
     if path.endswith(".lz4"):
         with open(path, "rb") as f:
             raw = lz4_stream_read(f)
     elif path.endswith(".gz"):
         with gzip.open(path, "rb") as f:
-            raw = f.read()
+            raw = bytearray(f.read())
     else:
         with open(path, "rb") as f:
-            raw = f.read()
+            raw = bytearray(f.read())
     return _decode(raw)
 
 

@@ -174,8 +174,9 @@ class Word2Vec:
             self._wm = dict(n=n, words=ibuf(n), lb=ibuf(n), ub=ibuf(n), ctx=ibuf(cap),
                             negs=ibuf(o.nneg * (cap // o.nreuse + 1)), counts=ibuf(2))
         b = self._wm
-        # the data source's 2 x n matrix, column-major: (word, sentence) pairs interleaved
-        dmats = torch.from_numpy(np.ascontiguousarray(wordsens.T.astype(np.int32))).to(self.device)
+        # the data source's 2 x n matrix, column-major: (word, sentence) pairs interleaved (no copy
+        # on the host if it already is, as matio.loadIMat returns it)
+        dmats = torch.from_numpy(np.ascontiguousarray(wordsens.T, dtype=np.int32)).to(self.device)
         self._call += 1
         npairs, ngroups = _device_wordmats(n, dmats, o.iflip, o.vocabSize, o.nskip, o.nneg,
                                            o.nreuse, float(np.float32(self.salpha)), o.wexpt,
@@ -191,15 +192,24 @@ class Word2Vec:
         return tuple(self._dev(x) for x in self.wordMats(mats))
 
     # ---- the four dispatchers (Word2Vec.scala:366-402, 469-523) --------------------------
+    # The update calls are enqueued without waiting (the Async entry points): the host then
+    # prepares the next minibatch while the device works.  Everything that reads the model
+    # afterwards (the scoring calls, torch on the same stream, synchronize()) is ordered behind
+    # them.
     def procPositives(self, nskip, words, lb, ub, model1, model2, lrate, vexp):
         nrows = model1.shape[1]
-        check(CUMACH.word2vecPos(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
-                                 lrate, vexp), "word2vecPos")
+        check(CUMACH.word2vecPosAsync(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
+                                      lrate, vexp), "word2vecPos")
 
     def procNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb, lrate, vexp):
         nrows = modela.shape[1]
-        check(CUMACH.word2vecNeg(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb, modela,
-                                 modelb, lrate, vexp), "word2vecNeg")
+        check(CUMACH.word2vecNegAsync(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
+                                      modela, modelb, lrate, vexp), "word2vecNeg")
+
+    def synchronize(self):
+        """Waits for the enqueued updates and raises if any of them failed."""
+        from .cumach import synchronize
+        synchronize()
 
     def evalPositives(self, nskip, words, lb, ub, model1, model2):
         nrows = model1.shape[1]
@@ -318,7 +328,7 @@ class Word2Vec:
             if m.shape[0] != self.opts.dim:
                 raise ValueError("modelmat%02d has %d rows, the model's dim is %d"
                                  % (len(mats), m.shape[0], self.opts.dim))
-            mats.append(np.array(m.T, order="C", copy=True))     # loadMat's buffer is read-only
+            mats.append(np.ascontiguousarray(m.T))
         if len(mats) < 2 or len(mats) % 2:
             raise ValueError("no model matrices under %r" % fname)
         self.init(self.ncols, modelmats=mats)
@@ -345,4 +355,5 @@ class Word2Vec:
                 else:
                     self.dobatch(mats, ipass, here)
                 istep += 1
+        self.synchronize()
         return results
