@@ -28,20 +28,29 @@
 namespace w2v {
 
 // Forward-only twin: sum over the group's pairs of log(max(1 - sigmoid(s), floor)).
+// Persistent: workgroup b walks groups [b*groups_per_wg, (b+1)*groups_per_wg), one group per wave
+// at a time, and a wave fetches the word ids of its next group while it works on the current
+// one, so that the only memory latency left on its critical path is that of the column gathers.
 template <int R, int MAXB, int CHA>
 __global__ void __launch_bounds__(kBlock)
-neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int* __restrict__ WA,
-                const int* __restrict__ WB, const float* __restrict__ A,
-                const float* __restrict__ B, double floorv, double* __restrict__ partials) {
+neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
+                const int* __restrict__ WA, const int* __restrict__ WB,
+                const float* __restrict__ A, const float* __restrict__ B, double floorv,
+                double* __restrict__ partials) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t unit = xcd_contiguous_block(per_xcd) * kWavesPerBlock + wave;
+  const int64_t g_begin = (int64_t)blockIdx.x * groups_per_wg;
+  const int64_t g_end = min(g_begin + groups_per_wg, (int64_t)ngroups);
   double lsum = 0.0;
 
-  if (unit < ngroups) {
-    int wbl = -1;
+  int64_t unit = g_begin + wave;
+  int wbl = -1, wal0 = -1;
+  if (unit < g_end) {
     if (lane < nwb) wbl = WB[unit * nwb + lane];
+    if (lane < nwa) wal0 = WA[unit * nwa + lane];
+  }
+  for (; unit < g_end; unit += kWavesPerBlock) {
     float b[MAXB][R];
     int wb[MAXB];
 #pragma unroll
@@ -52,9 +61,19 @@ neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int
         if (wb[k] >= 0) load_col<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
       }
     }
+    // ids of this wave's next group, in flight while this group is scored
+    const int64_t next = unit + kWavesPerBlock;
+    int wbl_next = -1, wal_next = -1;
+    if (next < g_end) {
+      if (lane < nwb) wbl_next = WB[next * nwb + lane];
+      if (lane < nwa) wal_next = WA[next * nwa + lane];
+    }
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
-      int wal = -1;
-      if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
+      int wal = wal0;
+      if (jbase > 0) {
+        wal = -1;
+        if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
+      }
       const int jend = min(nwa - jbase, kWave);
       for (int j0 = 0; j0 < jend; j0 += CHA) {
         float a[CHA][R];
@@ -87,9 +106,13 @@ neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t per_xcd, const int
         if (live) lsum += log(fmax(1.0 - (double)sat_sigmoid(pre), floorv));
       }
     }
+    wbl = wbl_next;
+    wal0 = wal_next;
   }
   block_store_partial(wave_sum_f64(lsum), partials);
 }
+
+constexpr int64_t kMinEvalGroupsPerWg = 64;
 
 constexpr int kNegWaves = 4;
 constexpr int kNegThreads = kNegWaves * kWave;
@@ -216,11 +239,19 @@ struct NegChunk {
 template <int R, int MAXB>
 static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int nwa, int nwb,
                                      const int* WA, const int* WB, float* A, float* B,
-                                     double floorv, double* partials) {
-  const int64_t per_xcd = blocks_per_xcd(ngroups);
-  const dim3 grid((unsigned)(per_xcd * kXcds));
-  hipLaunchKernelGGL((neg_eval_kernel<R, MAXB, NegChunk<R, MAXB>::value>), grid, dim3(kBlock), 0,
-                     stream, d, ngroups, nwa, nwb, per_xcd, WA, WB, A, B, floorv, partials);
+                                     double floorv, double* partials, int64_t* nparts) {
+  auto kern = neg_eval_kernel<R, MAXB, NegChunk<R, MAXB>::value>;
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, ngroups,
+                                   kMinEvalGroupsPerWg, &nwg);
+  if (err != hipSuccess) return err;
+  const int64_t cap = eval_partials_needed(ngroups);   // what the caller's buffer holds
+  if (nwg > cap) nwg = cap;
+  const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
+  nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
+                     groups_per_wg, WA, WB, A, B, floorv, partials);
+  *nparts = nwg;
   return hipGetLastError();
 }
 
@@ -247,12 +278,13 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
 template <int R, bool TRAIN>
 static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
                                const int* WA, const int* WB, float* A, float* B, float lrate,
-                               float vexp, double floorv, double* partials, Shadow shadow) {
+                               float vexp, double floorv, double* partials, int64_t* nparts,
+                               Shadow shadow) {
 #define W2V_NEG_DISPATCH(MAXB_)                                                                  \
   return TRAIN ? launch_neg_train_rb<R, MAXB_>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, A, \
                                                B, lrate, vexp, shadow)                           \
                : launch_neg_eval_rb<R, MAXB_>(stream, d, ngroups, nwa, nwb, WA, WB, A, B, floorv, \
-                                              partials)
+                                              partials, nparts)
   if (nwb <= 2) W2V_NEG_DISPATCH(2);
   if (nwb <= 5) W2V_NEG_DISPATCH(5);
   if (nwb <= kMaxNwb) W2V_NEG_DISPATCH(kMaxNwb);
@@ -264,9 +296,10 @@ hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int
                       const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
                       Shadow shadow) {
   const int rounds = (nrows + kWave - 1) / kWave;
+  int64_t unused = 0;
 #define CALL(R)                                                                                   \
   return launch_neg_r<R, true>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp, \
-                               0.0, nullptr, shadow)
+                               0.0, nullptr, &unused, shadow)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }
@@ -276,14 +309,16 @@ hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, in
                            double floorv, double* partials, float* Retval32, double* Retval64) {
   const int rounds = (nrows + kWave - 1) / kWave;
   hipError_t err = hipSuccess;
+  int64_t nparts = 0;
 #define CALL(R)                                                                                   \
   err = launch_neg_r<R, false>(stream, nrows, ncols, 0, nwa, nwb, WA, WB, const_cast<float*>(A),  \
-                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials, Shadow{});    \
+                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials, &nparts,      \
+                               Shadow{});                                                         \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
   if (err != hipSuccess) return err;
-  return launch_finalize(stream, partials, eval_partials_needed(ncols), Retval32, Retval64);
+  return launch_finalize(stream, partials, nparts, Retval32, Retval64);
 }
 
 }  // namespace w2v
