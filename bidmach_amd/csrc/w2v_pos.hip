@@ -7,12 +7,12 @@
 //   B[:,W[i+j]] += bscale * g * A[:,W[i]]
 //   A[:,W[i]]   += ascale * g * B[:,W[i+j]]    (accumulated over the window, scattered once)
 //
-// Two kernels.
+// Three kernels.
 //
-// pos_kernel (forward-only scoring, and the update when a tile does not fit in LDS): one
-// wavefront owns one centre token.  Its A column stays in registers for the whole window;
-// context columns are gathered CH at a time (all loads of a chunk are issued before the first
-// dot product, so a wave keeps CH columns in flight), dot products are reduced with DPP row
+// pos_kernel (the update when a tile does not fit in LDS) and pos_eval_kernel (forward-only
+// scoring): one wavefront owns one centre token.  Its A column stays in registers for the whole
+// window; context columns are gathered CH at a time (all loads of a chunk are issued before the
+// first dot product, so a wave keeps CH columns in flight), dot products are reduced with DPP row
 // rotations, and the CH pre-activations are parked in lanes 0..CH-1 so that the sigmoid (a double
 // exp) is evaluated once per chunk instead of once per pair.
 //
@@ -127,6 +127,89 @@ pos_kernel(int d, int ncols, int64_t per_xcd, const int* __restrict__ W,
     block_store_partial(wsum, partials);
   }
 }
+
+// Forward-only scoring, persistent form of pos_kernel: workgroup b walks a contiguous range of
+// centres (ranges are laid out so that each XCD's workgroups cover one contiguous stretch of the
+// minibatch and neighbouring centres' shared context columns meet in one L2), one centre per wave
+// at a time, and a wave fetches word id and window bounds of its next centre while it scores the
+// current one.
+template <int R, int CH>
+__global__ void __launch_bounds__(kBlock)
+pos_eval_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ W,
+                const int* __restrict__ LB, const int* __restrict__ UB,
+                const float* __restrict__ A, const float* __restrict__ B, double floorv,
+                double* __restrict__ partials) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t per_xcd = gridDim.x / kXcds;   // the grid is a multiple of the XCD count
+  const int64_t range = xcd_contiguous_block(per_xcd);
+  const int64_t u_begin = range * units_per_wg;
+  const int64_t u_end = min(u_begin + units_per_wg, (int64_t)ncols);
+  double lsum = 0.0;
+
+  int64_t unit = u_begin + wave;
+  int wi = -1, lb = 0, ub = 0;
+  if (unit < u_end) {
+    wi = W[unit];
+    lb = LB[unit];
+    ub = UB[unit];
+  }
+  for (; unit < u_end; unit += kWavesPerBlock) {
+    const int i = (int)unit;
+    const int wi_now = __builtin_amdgcn_readfirstlane(wi);
+    const int jlo = max(__builtin_amdgcn_readfirstlane(lb), -i);
+    const int jhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 1 - i);
+    {
+      const int64_t next = unit + kWavesPerBlock;
+      wi = -1;
+      if (next < u_end) {
+        wi = W[next];
+        lb = LB[next];
+        ub = UB[next];
+      }
+    }
+    if (wi_now < 0) continue;
+    float a[R];
+    load_col<R>(a, A + (int64_t)wi_now * d, lane, d);
+    for (int base = jlo; base <= jhi; base += kWave) {
+      const int j = base + lane;
+      int wl = -1;
+      if (j <= jhi && j != 0) wl = W[i + j];
+      unsigned long long mask = __ballot(wl >= 0);
+      while (mask != 0ull) {
+        int src[CH];
+        int n = 0;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (mask != 0ull) {
+            src[c] = __builtin_ctzll(mask);
+            mask &= mask - 1ull;
+            n = c + 1;
+          } else {
+            src[c] = -1;
+          }
+        }
+        float b[CH][R];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (c < n) load_col<R>(b[c], B + (int64_t)read_lane(wl, src[c]) * d, lane, d);
+        }
+        float pre = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (c < n) {
+            const float s = wave_sum(dot_partial<R>(a, b[c]));
+            pre = (lane == c) ? s : pre;
+          }
+        }
+        if (lane < n) lsum += log(fmax((double)sat_sigmoid(pre), floorv));
+      }
+    }
+  }
+  block_store_partial(wave_sum_f64(lsum), partials);
+}
+
+constexpr int64_t kMinEvalCentresPerWg = 256;
 
 constexpr int kTileWaves = 8;
 constexpr int kTileThreads = kTileWaves * kWave;
@@ -614,19 +697,38 @@ hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, floa
   return hipGetLastError();
 }
 
+template <int R>
+static hipError_t launch_pos_eval_r(hipStream_t stream, int d, int ncols, const int* W,
+                                    const int* LB, const int* UB, const float* A, const float* B,
+                                    double floorv, double* partials, int64_t* nparts) {
+  auto kern = pos_eval_kernel<R, PosChunk<R>::value>;
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, ncols,
+                                   kMinEvalCentresPerWg, &nwg);
+  if (err != hipSuccess) return err;
+  const int64_t cap = eval_partials_needed(ncols);   // what the caller's buffer holds
+  if (nwg > cap) nwg = cap;
+  nwg = (nwg + kXcds - 1) / kXcds * kXcds;           // whole XCD rows; empty ranges write 0
+  const int64_t units_per_wg = ((int64_t)ncols + nwg - 1) / nwg;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, units_per_wg, W,
+                     LB, UB, A, B, floorv, partials);
+  *nparts = nwg;
+  return hipGetLastError();
+}
+
 hipError_t launch_eval_pos(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
                            const int* UB, const float* A, const float* B, double floorv,
                            double* partials, float* Retval32, double* Retval64) {
   const int rounds = (nrows + kWave - 1) / kWave;
   hipError_t err = hipSuccess;
-#define CALL(R)                                                                                  \
-  err = launch_pos_r<R, false>(stream, nrows, ncols, W, LB, UB, const_cast<float*>(A),           \
-                               const_cast<float*>(B), 0.0f, 0.0f, floorv, partials);             \
+  int64_t nparts = 0;
+#define CALL(R)                                                                              \
+  err = launch_pos_eval_r<R>(stream, nrows, ncols, W, LB, UB, A, B, floorv, partials, &nparts); \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
   if (err != hipSuccess) return err;
-  return launch_finalize(stream, partials, eval_partials_needed(ncols), Retval32, Retval64);
+  return launch_finalize(stream, partials, nparts, Retval32, Retval64);
 }
 
 }  // namespace w2v
