@@ -71,7 +71,7 @@ extern "C" {
 size_t w2v_lz4_compress_bound(size_t n) { return n + n / 255 + 16; }
 
 long long w2v_lz4_compress(const void* src_, size_t n, void* dst_, size_t cap) {
-  if ((!src_ && n) || !dst_) return -1;
+  if ((!src_ && n) || !dst_ || n > 0x7fffffffu) return -1;
   const uint8_t* const src = static_cast<const uint8_t*>(src_);
   uint8_t* const dst = static_cast<uint8_t*>(dst_);
   uint8_t* op = dst;
@@ -80,15 +80,15 @@ long long w2v_lz4_compress(const void* src_, size_t n, void* dst_, size_t cap) {
   const uint8_t* anchor = src;
 
   if (n >= (size_t)kMatchSafeguard + 1) {
-    static thread_local int64_t table[1 << kHashBits];
+    int32_t table[1 << kHashBits];  // last position seen for each hash, 64 KB on the stack
     for (int i = 0; i < (1 << kHashBits); ++i) table[i] = -1;
     const uint8_t* const mflimit = iend - kMatchSafeguard;   // last position a match may start at
     const uint8_t* const matchlimit = iend - kLastLiterals;  // a match may not run past this
     const uint8_t* ip = src;
     while (ip <= mflimit) {
       const uint32_t h = hash4(read32(ip));
-      const int64_t cand = table[h];
-      table[h] = ip - src;
+      const int32_t cand = table[h];
+      table[h] = (int32_t)(ip - src);
       if (cand >= 0 && (size_t)((ip - src) - cand) <= kMaxOffset &&
           read32(src + cand) == read32(ip)) {
         const uint8_t* ref = src + cand;

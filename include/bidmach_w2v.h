@@ -193,7 +193,8 @@ const char *w2v_error_string(int err);
  * It stands in for the codec BIDMat reaches through lz4-java (both out of the reference tree) and
  * implements the published LZ4 block format; the stream framing is done by the caller.
  * compress/decompress return the number of bytes written, or -1 (output too small, or malformed
- * input); w2v_lz4_compress_bound(n) bytes of output always suffice to compress n bytes. */
+ * input, or more than 2^31 - 1 bytes to compress); w2v_lz4_compress_bound(n) bytes of output always
+ * suffice to compress n bytes. */
 size_t w2v_lz4_compress_bound(size_t n);
 long long w2v_lz4_compress(const void *src, size_t n, void *dst, size_t capacity);
 long long w2v_lz4_decompress(const void *src, size_t n, void *dst, size_t capacity);
