@@ -334,6 +334,22 @@ def main():
                                  "uploaded_bytes_per_step": upload}
         assert bool(torch.isfinite(A).all()) and bool(torch.isfinite(B).all()), "tables diverged"
 
+    # The streaming ceiling of this box, for scale: a plain 1 GiB device-to-device copy.
+    src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    copy_gbps = 5 * 2 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+    out["hbm_copy"] = {"achieved": copy_gbps, "unit": "GB/s read+write",
+                       "step_algorithmic_over_copy": step_gbps / copy_gbps}
+
     if not args.no_cpu_baseline and not evaluating:
         threads = host_threads()
         sample = host_mbs[:3]
