@@ -185,14 +185,16 @@ constexpr int kCounterStride = 32;  // one write counter per 128-byte line
 
 enum HotMode : int { kHotExact = 0, kHotCombining = 1, kHotOff = 2 };
 constexpr int kHotShareDen = 16;  // shadows are used if >= 1/16 of a launch's ids are hot words
+constexpr int kHotCountSlots = 256;  // blocks of the counting kernel, one partial count each
 
 struct Shadow {
   float* a;         // [kShadows][kHotWords][d] for table A
   float* b;         // same for table B
   unsigned* count;  // [2][kShadows][kHotWords][kCounterStride] write counters (B then A); they
                     // only ever count up, so they need no clearing between calls
-  int* hot_seen;        // how many of the launch's `hot_total` word ids are below kHotWords,
-  long long hot_total;  // counted on the device before the launch; hot_total == 0: not counted
+  int* hot_seen;        // kHotCountSlots partial counts: how many of the launch's `hot_total` word
+  long long hot_total;  // ids are below kHotWords, counted on the device before the launch;
+                        // hot_total == 0: not counted
   int combine;          // kHotExact or kHotCombining (kHotOff once resolved in a kernel)
 };
 
@@ -201,7 +203,11 @@ struct Shadow {
 // read and updated in place.
 __device__ __forceinline__ Shadow resolve_hot_mode(Shadow sh) {
   if (sh.hot_total > 0) {
-    const long long seen = __builtin_amdgcn_readfirstlane(*sh.hot_seen);
+    int part = 0;
+    for (int k = threadIdx.x & 63; k < kHotCountSlots; k += kWave) part += sh.hot_seen[k];
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) part += __shfl_xor(part, m, kWave);
+    const long long seen = __builtin_amdgcn_readfirstlane(part);
     if (seen * kHotShareDen < sh.hot_total) sh.combine = kHotOff;
   }
   return sh;

@@ -22,8 +22,9 @@ namespace w2v {
 // max_rows() floats.  The caller of launch_pos / launch_neg provides both buffers zeroed; the
 // launchers leave them zeroed.
 size_t shadow_bytes();
-// Bytes of the write counters of both tables' shadow copies plus the hot-word count of a launch
-// (zero-initialised once; the counters are never cleared, the count is cleared by launch_fold).
+// Bytes of the write counters of both tables' shadow copies plus the partial hot-word counts of a
+// launch (zero-initialised once; the counters are never cleared, the counts are rewritten by every
+// counting launch).
 size_t shadow_counter_bytes();
 
 // Grid size of a persistent kernel: the workgroups that fit on the device at once, but no more

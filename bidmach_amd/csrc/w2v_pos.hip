@@ -433,32 +433,46 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
   float* const table = blockIdx.y == 0 ? A : B;
   float* const sh = blockIdx.y == 0 ? shadow.a : shadow.b;
   for (int e = threadIdx.x; e < d; e += kBlock) {
+    float v[kShadows];
+#pragma unroll
+    for (int s = 0; s < kShadows; ++s) v[s] = sh[((int64_t)s * kHotWords + w) * d + e];  // all in flight
     float sum = 0.0f;
     bool any = false;
 #pragma unroll
     for (int s = 0; s < kShadows; ++s) {
-      float* p = sh + ((int64_t)s * kHotWords + w) * d + e;
-      const float v = *p;
-      if (v != 0.0f) {
+      if (v[s] != 0.0f) {
         any = true;
-        sum += v;
-        *p = 0.0f;
+        sum += v[s];
+        sh[((int64_t)s * kHotWords + w) * d + e] = 0.0f;
       }
     }
     if (any) table[(int64_t)w * d + e] += sum;
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *shadow.hot_seen = 0;
 }
 
-// Counts the word ids below kHotWords into *out (zero before the launch): one atomic per block,
-// so the adds to the one counter do not queue up.
+// Counts the word ids below kHotWords: block b leaves its share in out[b] (kHotCountSlots blocks,
+// every slot is written on every launch, so nothing needs clearing and no atomics queue up).
 __global__ void __launch_bounds__(kBlock)
-count_hot_kernel(const int* __restrict__ ids, int64_t n, int* out) {
+count_hot_kernel(const int* __restrict__ ids, int64_t n, int* __restrict__ out) {
   __shared__ int s_part[kWavesPerBlock];
   int local = 0;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    const int w = ids[i];
-    local += (w >= 0 && w < kHotWords) ? 1 : 0;
+  const int64_t n4 = n / 4;
+  const int4* ids4 = reinterpret_cast<const int4*>(ids);   // device allocations are 16-byte aligned
+  const bool aligned = (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
+  auto hot = [](int w) { return (w >= 0 && w < kHotWords) ? 1 : 0; };
+  if (aligned) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4;
+         i += (int64_t)gridDim.x * kBlock) {
+      const int4 v = ids4[i];
+      local += hot(v.x) + hot(v.y) + hot(v.z) + hot(v.w);
+    }
+    for (int64_t i = n4 * 4 + (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * kBlock)
+      local += hot(ids[i]);
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * kBlock)
+      local += hot(ids[i]);
   }
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) local += __shfl_xor(local, m, kWave);
@@ -468,13 +482,14 @@ count_hot_kernel(const int* __restrict__ ids, int64_t n, int* out) {
     int total = 0;
 #pragma unroll
     for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
-    if (total != 0) atomicAdd(out, total);
+    out[blockIdx.x] = total;
   }
 }
 
 size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
 size_t shadow_counter_bytes() {
-  return ((size_t)2 * kShadows * kHotWords + 1) * kCounterStride * sizeof(unsigned);
+  return (size_t)2 * kShadows * kHotWords * kCounterStride * sizeof(unsigned) +
+         (size_t)kHotCountSlots * sizeof(int);
 }
 
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d) {
@@ -508,9 +523,7 @@ hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64
   if (n <= 0) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
   // read the count from memory, the host does not wait for it).
-  const int64_t want = (n + 16 * kBlock - 1) / (16 * kBlock);
-  const unsigned grid = (unsigned)(want < 1 ? 1 : (want > 256 ? 256 : want));
-  hipLaunchKernelGGL(count_hot_kernel, dim3(grid), dim3(kBlock), 0, stream, ids, n,
+  hipLaunchKernelGGL(count_hot_kernel, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids, n,
                      shadow->hot_seen);
   shadow->hot_total = n;
   return hipGetLastError();
