@@ -124,9 +124,9 @@ def main():
     ap.add_argument("--wsample", type=float, default=0.0,
                     help="frequent-word subsampling threshold of the reference caller (its default "
                          "is 1e-4); 0 = the raw stream the headline metric is defined on")
-    ap.add_argument("--hot-mode", type=int, default=-1, choices=[-1, 0, 1],
+    ap.add_argument("--hot-mode", type=int, default=-1, choices=[-1, 0, 1, 2],
                     help="w2v_set_hot_update_mode: -1 the library's per-launch choice (default), "
-                         "0 exact shadow copies, 1 combining shadow copies")
+                         "0 exact shadow copies, 1 combining shadow copies, 2 no shadow copies")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")

@@ -502,7 +502,7 @@ void set_max_workgroups(int n) { g_max_workgroups.store(n < 0 ? 0 : n); }
 int get_max_workgroups() { return g_max_workgroups.load(); }
 
 static std::atomic<int> g_hot_update_mode{-1};
-void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode == 0 || mode == 1 ? mode : -1); }
+void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode >= 0 && mode <= 2 ? mode : -1); }
 int get_hot_update_mode() { return g_hot_update_mode.load(); }
 
 // Chooses how a launch of nwg workgroups treats the hot words (Shadow::combine and the hot-word
@@ -515,7 +515,7 @@ hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64
                             int waves_per_wg, Shadow* shadow) {
   const int mode = g_hot_update_mode.load();
   shadow->hot_total = 0;
-  if (mode == kHotExact || mode == kHotCombining) {
+  if (mode == kHotExact || mode == kHotCombining || mode == kHotOff) {
     shadow->combine = mode;
     return hipSuccess;
   }

@@ -141,6 +141,7 @@ int w2v_get_max_workgroups(void);
  *      write to it, which hides fewer than 8 updates per copy (a couple of hundred of the most
  *      frequent word) from readers for a few microseconds; about 20 % faster than 0 on a raw
  *      Zipf stream;
+ *   2  off: no shadow copies, every column is read and updated in place;
  *  -1  (default) decided per launch on the device: no shadow copies at all unless at least 1/16
  *      of the launch's word ids are among those 16 (they are not after frequent-word subsampling);
  *      otherwise combining for launches with at least 2048 wavefronts in flight, where that many

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 gpu = parity.gpu
 
 
-@pytest.fixture(params=[0, 1], ids=["exact", "combining"])
+@pytest.fixture(params=[0, 1, 2], ids=["exact", "combining", "off"])
 def hot_mode(request):
     from bidmach_amd.cumach import load_library
     lib = load_library()
@@ -78,7 +78,7 @@ def test_hot_columns_receive_every_update_exactly_once(gpu, hot_mode):
 def test_mode_argument_is_normalised(gpu):
     from bidmach_amd.cumach import load_library
     lib = load_library()
-    for given, kept in ((7, -1), (1, 1), (0, 0), (-5, -1)):
+    for given, kept in ((7, -1), (1, 1), (0, 0), (2, 2), (-5, -1)):
         lib.w2v_set_hot_update_mode(given)
         assert lib.w2v_get_hot_update_mode() == kept
     lib.w2v_set_hot_update_mode(-1)
