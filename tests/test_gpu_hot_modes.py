@@ -45,16 +45,17 @@ def test_sliced_model(gpu, oracle, hot_mode):
     sliced.test_colliding_minibatch_stays_close_to_sequential_oracle(gpu, oracle)
 
 
-def test_hot_columns_receive_every_update_exactly_once(gpu, hot_mode):
+@pytest.mark.parametrize("d", [37, 128, 300, 1280])
+def test_hot_columns_receive_every_update_exactly_once(gpu, hot_mode, d):
     """Only words 0..15, tens of thousands of updates each, with the A table zero: every B delta
     is then lr * 0.5 * 0 = 0 and every A delta is the sum of -lr/2 * B columns, known exactly up
     to rounding whatever the interleaving.  Shadow copies that lost or duplicated a write, or a
     fold that dropped what it swapped out, would show as a wrong multiple."""
     torch, CUMACH = gpu
     rng = np.random.default_rng(4)
-    d, V, G, nwa, nwb = 128, 64, 60000, 5, 5
+    V, G, nwa, nwb = 64, (60000 if d <= 300 else 12000), 5, 5
     A = np.zeros((V, d), np.float32)
-    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1 * (128.0 / d) ** 0.5).astype(np.float32)
     WA = rng.integers(0, 16, G * nwa).astype(np.int32)
     WB = rng.integers(0, 16, G * nwb).astype(np.int32)
     lr = 1e-6
