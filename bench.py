@@ -121,6 +121,9 @@ def main():
                          "this process is worker 0 and holds only its share of the model")
     ap.add_argument("--head", type=int, default=0,
                     help="with --parts: number of head words (resident on every worker)")
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="tokens per minibatch, overriding the workload's (the reference's own "
+                         "default minibatch is 100000 tokens)")
     ap.add_argument("--wsample", type=float, default=0.0,
                     help="frequent-word subsampling threshold of the reference caller (its default "
                          "is 1e-4); 0 = the raw stream the headline metric is defined on")
@@ -146,7 +149,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     from bidmach_amd.cumach import load_library
     load_library().w2v_set_hot_update_mode(args.hot_mode)
-    cfg = WORKLOADS[args.workload]
+    cfg = dict(WORKLOADS[args.workload])
+    if args.tokens > 0:
+        cfg["tokens"] = args.tokens
     d, V, n = cfg["dim"], cfg["vocab"], cfg["tokens"]
     K, Wm = args.steps, args.warmup
 

@@ -213,6 +213,12 @@ __device__ __forceinline__ Shadow resolve_hot_mode(Shadow sh) {
   return sh;
 }
 
+// True if the launch counted its hot words and found too few: such a launch has no column that a
+// large share of the units in flight would update, so it may spread over the whole device.
+__device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow& resolved) {
+  return asked.hot_total > 0 && asked.combine != kHotOff && resolved.combine == kHotOff;
+}
+
 __device__ __forceinline__ int shadow_copies(int w, int combine) {
   const int c = (combine == kHotCombining ? kShadows : kShadowsExact) >> (31 - __builtin_clz(w + 1));
   return c < 2 ? 2 : c;

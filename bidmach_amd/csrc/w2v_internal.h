@@ -31,6 +31,12 @@ size_t shadow_counter_bytes();
 // than `units / min_units_per_wg` (a workgroup walks at least that many work units, so a small
 // minibatch is not spread over the whole device: fewer units in flight means less stale Hogwild
 // updates), and no more than the caller's limit (set_max_workgroups, 0 = none).
+struct GridSplit {
+  int64_t nwg, per_wg;            // bounded grid: workgroups and units per workgroup
+  int64_t nwg_wide, per_wg_wide;  // device-filling grid (never smaller than the bounded one)
+};
+hipError_t split_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
+                      int64_t min_units, int64_t min_units_wide, GridSplit* out);
 hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
                            int64_t min_units_per_wg, int64_t* nwg);
 void set_max_workgroups(int n);

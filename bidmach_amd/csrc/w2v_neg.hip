@@ -117,6 +117,7 @@ constexpr int64_t kMinEvalGroupsPerWg = 64;
 constexpr int kNegWaves = 4;
 constexpr int kNegThreads = kNegWaves * kWave;
 constexpr int kMinGroupsPerWg = 512;  // a workgroup walks at least this many consecutive groups
+constexpr int kMinGroupsPerWgWide = 32;  // the same for a launch without hot words
 // Waves per SIMD the update kernel is compiled for.  The pass is bound by atomic latency, so it
 // wants waves in flight more than it wants registers per wave.
 #ifndef W2V_NEG_WAVES_PER_EU
@@ -125,7 +126,8 @@ constexpr int kMinGroupsPerWg = 512;  // a workgroup walks at least this many co
 
 template <int R, int MAXB, int CHA>
 __global__ void __launch_bounds__(kNegThreads, W2V_NEG_WAVES_PER_EU)
-neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t groups_per_wg,
+neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t groups_per_wg_hot,
+                 int64_t groups_per_wg_wide,
                  const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
                  float lrate, float vexp, int smode, Shadow shadow_arg) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
@@ -134,6 +136,8 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
+  const int64_t groups_per_wg = launch_is_cold(shadow_arg, shadow) ? groups_per_wg_wide
+                                                                    : groups_per_wg_hot;
   const int64_t g_begin = (int64_t)blockIdx.x * groups_per_wg;
   const int64_t g_end = min(g_begin + groups_per_wg, (int64_t)ngroups);
 
@@ -260,16 +264,17 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
                                       int nwb, const int* WA, const int* WB, float* A, float* B,
                                       float lrate, float vexp, Shadow shadow) {
   auto kern = neg_train_kernel<R, MAXB, NegChunk<R, MAXB>::value>;
-  int64_t nwg = 0;
-  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, ngroups,
-                                   kMinGroupsPerWg, &nwg);
+  GridSplit g;
+  hipError_t err = split_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, ngroups,
+                              kMinGroupsPerWg, kMinGroupsPerWgWide, &g);
   if (err != hipSuccess) return err;
-  const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
-  nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
-  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nwg, kNegWaves, &shadow);
+  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, g.nwg, kNegWaves, &shadow);
   if (err != hipSuccess) return err;
+  // only a launch that counts its hot words can turn out cold
+  const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, idlimit,
-                     nwa, nwb, groups_per_wg, WA, WB, A, B, lrate, vexp, scale_mode(vexp), shadow);
+                     nwa, nwb, g.per_wg, g.per_wg_wide, WA, WB, A, B, lrate, vexp,
+                     scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
   return launch_fold(stream, A, B, shadow, d);

@@ -215,6 +215,7 @@ constexpr int kTileWaves = 8;
 constexpr int kTileThreads = kTileWaves * kWave;
 constexpr int kMaxHalo = 31;       // 2*Sh + 1 window offsets must fit in the 64 lanes of a wave
 constexpr int kMinTilesPerWg = 64; // a workgroup walks at least this many consecutive tiles
+constexpr int kMinTilesPerWgWide = 4;  // the same for a launch without hot words
 
 // LDS layout of a workgroup:
 //   a_t[T][dp] | b_t[T + 2*Sh][dp] | G[T][2*Sh + 1] | wt[T + 2*Sh] | ft[T + 2*Sh]
@@ -232,7 +233,8 @@ __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
 // budget is held to that.
 template <int R, class Tables>
 __global__ void __launch_bounds__(kTileThreads, (R <= 7 ? 4 : 2))
-pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg,
+pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg_hot,
+                int64_t tiles_per_wg_wide,
                 const int* __restrict__ W, const int* __restrict__ LB,
                 const int* __restrict__ UB, Tables tables, float lrate, float vexp, int smode,
                 Shadow shadow_arg) {
@@ -249,6 +251,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
   int* const ft = wt + (T + 2 * Sh);
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
+  const int64_t tiles_per_wg = launch_is_cold(shadow_arg, shadow) ? tiles_per_wg_wide
+                                                                   : tiles_per_wg_hot;
   const int64_t tile_begin = (int64_t)blockIdx.x * tiles_per_wg;
   const int64_t tile_end = min(tile_begin + tiles_per_wg, ntiles);
 
@@ -549,6 +553,32 @@ hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, in
   return hipSuccess;
 }
 
+// Two ways of cutting `units` over a persistent grid.  `bounded` gives every workgroup at least
+// min_units consecutive units, which keeps the number of units in flight (whose updates do not see
+// each other) small against a launch that is full of frequent words; `wide` fills the device as
+// soon as every workgroup has min_units_wide units.  The kernel is launched with the wide grid and
+// picks one of the two once it knows whether the launch holds hot words.
+hipError_t split_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
+                      int64_t min_units, int64_t min_units_wide, GridSplit* out) {
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(kernel, threads, lds_bytes, units, min_units, &nwg);
+  if (err != hipSuccess) return err;
+  out->per_wg = (units + nwg - 1) / nwg;
+  if (out->per_wg < 1) out->per_wg = 1;
+  out->nwg = (units + out->per_wg - 1) / out->per_wg;
+  if (out->nwg < 1) out->nwg = 1;
+  err = persistent_grid(kernel, threads, lds_bytes, units, min_units_wide, &nwg);
+  if (err != hipSuccess) return err;
+  out->per_wg_wide = (units + nwg - 1) / nwg;
+  if (out->per_wg_wide < 1) out->per_wg_wide = 1;
+  out->nwg_wide = (units + out->per_wg_wide - 1) / out->per_wg_wide;
+  if (out->nwg_wide < out->nwg) {
+    out->nwg_wide = out->nwg;
+    out->per_wg_wide = out->per_wg;
+  }
+  return hipSuccess;
+}
+
 // Sum of the block's 256 per-thread values by a fixed LDS tree; the result is valid in thread 0.
 __device__ __forceinline__ double block_tree_sum(double t, double* s) {
   s[threadIdx.x] = t;
@@ -643,17 +673,17 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
     if (err != hipSuccess) return err;
   }
   const int64_t ntiles = ((int64_t)ncols + T - 1) / T;
-  int64_t nwg = 0;
-  err = persistent_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, ntiles,
-                        kMinTilesPerWg, &nwg);
+  GridSplit g;
+  err = split_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, ntiles, kMinTilesPerWg,
+                   kMinTilesPerWgWide, &g);
   if (err != hipSuccess) return err;
-  const int64_t tiles_per_wg = (ntiles + nwg - 1) / nwg;
-  nwg = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
-  err = prepare_hot_mode(stream, W, ncols, nwg, kTileWaves, &shadow);
+  err = prepare_hot_mode(stream, W, ncols, g.nwg, kTileWaves, &shadow);
   if (err != hipSuccess) return err;
+  // only a launch that counts its hot words can turn out cold
+  const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
-                     ntiles, tiles_per_wg, W, LB, UB, tables, lrate, vexp, scale_mode(vexp),
-                     shadow);
+                     ntiles, g.per_wg, g.per_wg_wide, W, LB, UB, tables, lrate, vexp,
+                     scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
   return launch_fold(stream, fold_a, fold_b, shadow, d);
