@@ -121,6 +121,9 @@ def main():
                          "this process is worker 0 and holds only its share of the model")
     ap.add_argument("--head", type=int, default=0,
                     help="with --parts: number of head words (resident on every worker)")
+    ap.add_argument("--rare-mode", type=int, default=-1, choices=(-1, 0, 1),
+                    help="w2v_set_rare_update_mode: 0 = float atomics for every column, -1/1 = "
+                         "plain read-modify-write for words that are rare within a call (default)")
     ap.add_argument("--tokens", type=int, default=0,
                     help="tokens per minibatch, overriding the workload's (the reference's own "
                          "default minibatch is 100000 tokens)")
@@ -149,6 +152,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     from bidmach_amd.cumach import load_library
     load_library().w2v_set_hot_update_mode(args.hot_mode)
+    load_library().w2v_set_rare_update_mode(args.rare_mode)
     cfg = dict(WORKLOADS[args.workload])
     if args.tokens > 0:
         cfg["tokens"] = args.tokens

@@ -53,7 +53,7 @@ hipError_t eval_scratch(int64_t need, double** out) {
 }
 
 // Per-thread, per-device shadow buffers for the hot columns and their write counters, allocated
-// and zeroed on first use: [shadow of A | shadow of B | counters].
+// and zeroed on first use: [shadow of A | shadow of B | counters | word occurrence counts].
 hipError_t shadow_buffers(w2v::Shadow* out) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -63,7 +63,7 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   const size_t bytes = w2v::shadow_bytes();
   if (ts.shadow[dev] == nullptr) {
     float* p = nullptr;
-    const size_t total = 2 * bytes + w2v::shadow_counter_bytes();
+    const size_t total = 2 * bytes + w2v::shadow_counter_bytes() + w2v::occurs_bytes();
     err = hipMalloc(reinterpret_cast<void**>(&p), total);
     if (err != hipSuccess) return err;
     err = hipMemsetAsync(p, 0, total, ts.stream);
@@ -79,6 +79,9 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   out->count = reinterpret_cast<unsigned*>(ts.shadow[dev] + 2 * (bytes / sizeof(float)));
   out->hot_seen = reinterpret_cast<int*>(out->count + (size_t)2 * w2v::kShadows * w2v::kHotWords *
                                                           w2v::kCounterStride);
+  out->occurs = reinterpret_cast<int*>(reinterpret_cast<char*>(out->count) +
+                                       w2v::shadow_counter_bytes());
+  out->rare_max = 0;
   out->hot_total = 0;
   out->combine = 0;
   return hipSuccess;
@@ -359,6 +362,12 @@ int w2v_set_max_workgroups(int n) {
   return 0;
 }
 int w2v_get_max_workgroups(void) { return w2v::get_max_workgroups(); }
+
+int w2v_set_rare_update_mode(int mode) {
+  w2v::set_rare_update_mode(mode);
+  return 0;
+}
+int w2v_get_rare_update_mode(void) { return w2v::get_rare_update_mode(); }
 
 int w2v_set_hot_update_mode(int mode) {
   w2v::set_hot_update_mode(mode);

@@ -140,6 +140,35 @@ __device__ __forceinline__ void atomic_add_col(float* __restrict__ col, const fl
   }
 }
 
+// The Hogwild update without atomic adds, for words that occur so rarely in a launch that two
+// updates of one column are practically never in flight together (see Shadow::occurs): the column
+// is read with load_col_fresh where other columns are read with load_col, and written back as
+// fresh + delta.  Both sides bypass the XCD-local L2 (device-scope loads and stores), because plain
+// stores of one XCD are not visible to the others while a kernel runs.  What other writers add
+// between the load and the store is overwritten.  Without a concurrent writer the result is
+// bit-identical to the atomic update.
+template <int R>
+__device__ __forceinline__ void load_col_fresh(float (&x)[R], const float* col, int lane, int d) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int e = r * kWave + lane;
+    x[r] = (r < R - 1 || e < d)
+               ? __hip_atomic_load(col + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+               : 0.0f;
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void store_sum_col(float* col, const float (&fresh)[R],
+                                              const float (&x)[R], int lane, int d) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int e = r * kWave + lane;
+    if (r < R - 1 || e < d)
+      __hip_atomic_store(col + e, fresh[r] + x[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 template <int R>
 __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float alpha,
                                                 const float (&x)[R], int lane, int d) {
@@ -196,7 +225,24 @@ struct Shadow {
   long long hot_total;  // ids are below kHotWords, counted on the device before the launch;
                         // hot_total == 0: not counted
   int combine;          // kHotExact or kHotCombining (kHotOff once resolved in a kernel)
+  // Rare words.  The float-atomic units are what bounds the update passes, and most of their work
+  // is spent on columns that are touched a handful of times per launch, where two updates of the
+  // same column are practically never in flight together.  occurs[w & (kOccurSlots - 1)] holds how
+  // often word w occurs in the launch (counted on the device beforehand, saturating just above
+  // rare_max; slots shared by several words only err towards atomics); a word with at most
+  // rare_max occurrences is updated with a plain read-modify-write.  rare_max == 0: every update
+  // is atomic.
+  int* occurs;
+  int rare_max;
 };
+
+constexpr int kOccurSlots = 1 << 20;
+
+// Whether word w (>= 0) of this launch is updated without atomics.  The words that may have
+// shadow copies never are.
+__device__ __forceinline__ bool is_rare(const Shadow& sh, int w) {
+  return sh.rare_max > 0 && w >= kHotWords && sh.occurs[w & (kOccurSlots - 1)] <= sh.rare_max;
+}
 
 // The mode a kernel runs in: the launcher's, unless the ids of this launch hold too few hot words
 // for shadow copies to pay (subsampled or re-numbered vocabularies), in which case every column is

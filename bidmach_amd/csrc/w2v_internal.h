@@ -48,6 +48,9 @@ int get_max_workgroups();
 // enqueues the count of hot words among them.
 void set_hot_update_mode(int mode);
 int get_hot_update_mode();
+void set_rare_update_mode(int mode);
+int get_rare_update_mode();
+size_t occurs_bytes();
 hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64_t nwg,
                             int waves_per_wg, Shadow* shadow);
 

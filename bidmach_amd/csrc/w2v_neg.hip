@@ -22,6 +22,8 @@
 //
 // The reference reads WA/WB without a validity test (:213-214,220-221); here a negative id
 // skips every pair it takes part in, so a bad id cannot become an out-of-bounds access.
+#include <atomic>
+
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
@@ -147,6 +149,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
     if (lane < nwb) wbl = WB[unit * nwb + lane];
     if (wbl >= idlimit) wbl = -1;  // word2vecNegFilt: ids beyond the resident columns are skipped
     const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
+    const uint64_t rare_b = __ballot(wbl >= 0 && is_rare(shadow, wbl));
     // tickets for the writes to hot B columns at the end of the group, taken now
     const unsigned tkb = hot_ticket(shadow, 0, slot, (wbl >= 0 && wbl < kHotWords) ? wbl : -1);
 
@@ -158,8 +161,12 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       wb[k] = -1;
       if (k < nwb) {
         wb[k] = read_lane(wbl, k);
-        if (wb[k] >= 0)
-          load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow.b, shadow.combine, lane, d);
+        if (wb[k] >= 0) {
+          if ((rare_b >> k) & 1)
+            load_col_fresh<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
+          else
+            load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow.b, shadow.combine, lane, d);
+        }
         zero_col<R>(dbb[k]);
       }
     }
@@ -169,6 +176,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
       if (wal >= idlimit) wal = -1;
       const float sal = wal >= 0 ? scale_of(wal, vexp, smode) : 0.0f;
+      const uint64_t rare_a = __ballot(wal >= 0 && is_rare(shadow, wal));
       const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
       const int jend = min(nwa - jbase, kWave);
 
@@ -180,8 +188,12 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
           wa[c] = -1;
           if (j0 + c < jend) {
             wa[c] = read_lane(wal, j0 + c);
-            if (wa[c] >= 0)
-              load_col_ref<R>(a[c], table_ref(A, wa[c], d), shadow.a, shadow.combine, lane, d);
+            if (wa[c] >= 0) {
+              if ((rare_a >> (j0 + c)) & 1)
+                load_col_fresh<R>(a[c], A + (int64_t)wa[c] * d, lane, d);
+              else
+                load_col_ref<R>(a[c], table_ref(A, wa[c], d), shadow.a, shadow.combine, lane, d);
+            }
           }
         }
         float pre = 0.0f;
@@ -213,8 +225,11 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
                 axpy<R>(daa, as * g, b[k]);
               }
             }
-            scatter_add_ref<R>(table_ref(A, wa[c], d), shadow, 1, slot, daa, lane, d,
-                               read_lane(tka, j0 + c));
+            if ((rare_a >> (j0 + c)) & 1)
+              store_sum_col<R>(A + (int64_t)wa[c] * d, a[c], daa, lane, d);
+            else
+              scatter_add_ref<R>(table_ref(A, wa[c], d), shadow, 1, slot, daa, lane, d,
+                                 read_lane(tka, j0 + c));
           }
         }
       }
@@ -222,11 +237,65 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
 
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
-      if (wb[k] >= 0)
-        scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d,
-                           read_lane(tkb, k));
+      if (wb[k] >= 0) {
+        if ((rare_b >> k) & 1)
+          store_sum_col<R>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d);
+        else
+          scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d,
+                             read_lane(tkb, k));
+      }
     }
   }
+}
+
+// Clears the occurrence counters (a kernel, not a memset, so that callers may capture the call).
+__global__ void __launch_bounds__(kBlock) clear_occurs_kernel(int4* __restrict__ p, int n4) {
+  for (int i = blockIdx.x * kBlock + threadIdx.x; i < n4; i += gridDim.x * kBlock)
+    p[i] = make_int4(0, 0, 0, 0);
+}
+
+// Counts how often each word occurs among the two id arrays of a launch, exactly up to rare_max
+// and saturating soon after: a slot that is already above rare_max is left alone, so the words that
+// occur hundreds of thousands of times do not queue that many atomics on one address.  Words that
+// may have shadow copies are never rare and are not counted.
+__global__ void __launch_bounds__(kBlock)
+count_occurs_kernel(const int* __restrict__ ids_a, int64_t na, const int* __restrict__ ids_b,
+                    int64_t nb, int idlimit, int* occurs, int rare_max) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < na + nb;
+       i += (int64_t)gridDim.x * kBlock) {
+    const int w = i < na ? ids_a[i] : ids_b[i - na];
+    if (w < kHotWords || w >= idlimit) continue;
+    int* const slot = occurs + (w & (kOccurSlots - 1));
+    if (__hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= rare_max)
+      __hip_atomic_fetch_add(slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+static std::atomic<int> g_rare_update_mode{-1};
+void set_rare_update_mode(int mode) { g_rare_update_mode.store(mode >= 0 ? mode : -1); }
+int get_rare_update_mode() { return g_rare_update_mode.load(); }
+
+// Decides how many occurrences still make a word of this launch "rare" and counts the words.  A
+// launch of `units` work units keeps `waves` of them in flight, so a word with n occurrences has
+// about n * waves / units updates in flight together; words for which that is below 1/16 are
+// updated without atomics.  Small launches get 0: everything stays atomic and nothing is counted.
+constexpr int kRareConcurrencyDen = 16;
+constexpr int kRareMaxCap = 64;
+static hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na,
+                                     const int* ids_b, int64_t nb, int idlimit, int64_t units,
+                                     int64_t waves, Shadow* shadow) {
+  shadow->rare_max = 0;
+  const int mode = g_rare_update_mode.load();
+  if (mode == 0 || shadow->occurs == nullptr || waves <= 0) return hipSuccess;
+  int64_t most = mode >= 2 ? mode : units / (kRareConcurrencyDen * waves);
+  if (most > kRareMaxCap) most = kRareMaxCap;
+  if (most < 1) return hipSuccess;
+  hipLaunchKernelGGL(clear_occurs_kernel, dim3(256), dim3(kBlock), 0, stream,
+                     reinterpret_cast<int4*>(shadow->occurs), kOccurSlots / 4);
+  hipLaunchKernelGGL(count_occurs_kernel, dim3(1024), dim3(kBlock), 0, stream, ids_a, na, ids_b, nb,
+                     idlimit, shadow->occurs, (int)most);
+  shadow->rare_max = (int)most;
+  return hipGetLastError();
 }
 
 constexpr int kMaxNwb = 8;
@@ -272,6 +341,9 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   if (err != hipSuccess) return err;
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;
+  err = prepare_rare_words(stream, WA, (int64_t)ngroups * nwa, WB, (int64_t)ngroups * nwb, idlimit,
+                           ngroups, nwg * kNegWaves, &shadow);
+  if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kNegThreads), 0, stream, d, ngroups, idlimit,
                      nwa, nwb, g.per_wg, g.per_wg_wide, WA, WB, A, B, lrate, vexp,
                      scale_mode(vexp), shadow);

@@ -496,6 +496,8 @@ size_t shadow_counter_bytes() {
          (size_t)kHotCountSlots * sizeof(int);
 }
 
+size_t occurs_bytes() { return (size_t)kOccurSlots * sizeof(int); }
+
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d) {
   hipLaunchKernelGGL(fold_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, shadow, d);
   return hipGetLastError();

@@ -61,6 +61,8 @@ SYMBOLS = {
     "w2v_get_max_workgroups": (_I, []),
     "w2v_set_hot_update_mode": (_I, [_I]),
     "w2v_get_hot_update_mode": (_I, []),
+    "w2v_set_rare_update_mode": (_I, [_I]),
+    "w2v_get_rare_update_mode": (_I, []),
     "w2v_max_rows": (_I, []),
     "w2v_max_nwb": (_I, []),
     "w2v_malloc": (_I, [ctypes.POINTER(_P), _SZ]),

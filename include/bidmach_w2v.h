@@ -149,6 +149,22 @@ int w2v_get_max_workgroups(void);
 int w2v_set_hot_update_mode(int mode);
 int w2v_get_hot_update_mode(void);
 
+/* How word2vecNeg / word2vecNegFilt update the columns of words that are rare within one call.
+ * No counterpart in the reference's GPU path, which uses atomicAdd throughout
+ * (jni/src/DNN127.cu:652-661); its CPU path updates every column with a plain read-modify-write from
+ * all threads (jni/src/BIDMach_CPUMACH.c:239-254).
+ *   0  every update is a float atomic;
+ *  -1, 1  (default) the call first counts, on the device, how often each word occurs in it; a word
+ *      with so few occurrences that fewer than 1/16 of an update of it is in flight at any time, on
+ *      average, is updated with a plain read-modify-write (bit-identical to the atomic update
+ *      unless two updates of that column do overlap, in which case one of them is lost, as on the
+ *      reference's CPU path).  Frequent words, and every word of a small call, stay atomic.  This
+ *      takes about a third of the load off the float-atomic units, which bound the pass.
+ *   n >= 2  (tests, experiments) words with at most min(n, 64) occurrences in the call are treated
+ *      that way whatever the size of the call. */
+int w2v_set_rare_update_mode(int mode);
+int w2v_get_rare_update_mode(void);
+
 /* Limits of the kernels: largest nrows and largest nwb. */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
