@@ -53,7 +53,8 @@ hipError_t eval_scratch(int64_t need, double** out) {
 }
 
 // Per-thread, per-device shadow buffers for the hot columns and their write counters, allocated
-// and zeroed on first use: [shadow of A | shadow of B | counters | word occurrence counts].
+// and zeroed on first use: [shadow of A | shadow of B | counters | word occurrence counts | read
+// copies of A | read copies of B].
 hipError_t shadow_buffers(w2v::Shadow* out) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -63,7 +64,8 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   const size_t bytes = w2v::shadow_bytes();
   if (ts.shadow[dev] == nullptr) {
     float* p = nullptr;
-    const size_t total = 2 * bytes + w2v::shadow_counter_bytes() + w2v::occurs_bytes();
+    const size_t total = 2 * bytes + w2v::shadow_counter_bytes() + w2v::occurs_bytes() +
+                         2 * w2v::read_copy_bytes();
     err = hipMalloc(reinterpret_cast<void**>(&p), total);
     if (err != hipSuccess) return err;
     err = hipMemsetAsync(p, 0, total, ts.stream);
@@ -82,6 +84,10 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   out->occurs = reinterpret_cast<int*>(reinterpret_cast<char*>(out->count) +
                                        w2v::shadow_counter_bytes());
   out->rare_max = 0;
+  out->hot_mask = out->hot_seen + w2v::kHotCountSlots;
+  out->pub_a = reinterpret_cast<float*>(reinterpret_cast<char*>(out->occurs) + w2v::occurs_bytes());
+  out->pub_b = out->pub_a + w2v::read_copy_bytes() / sizeof(float);
+  out->xcc = 0;
   out->hot_total = 0;
   out->combine = 0;
   return hipSuccess;

@@ -234,6 +234,12 @@ struct Shadow {
   // is atomic.
   int* occurs;
   int rare_max;
+  // Read copies of the hot columns for the combining mode: [kXcds][kHotWords][d] per table, one
+  // per XCD, or null (then readers read the table).  See load_col_ref.
+  float* pub_a;
+  float* pub_b;
+  int* hot_mask;  // [2][kHotCountSlots] partial bit masks of the hot ids seen: table B's, then A's
+  int xcc;        // the XCD this wave runs on (filled in by resolve_hot_mode)
 };
 
 constexpr int kOccurSlots = 1 << 20;
@@ -247,7 +253,13 @@ __device__ __forceinline__ bool is_rare(const Shadow& sh, int w) {
 // The mode a kernel runs in: the launcher's, unless the ids of this launch hold too few hot words
 // for shadow copies to pay (subsampled or re-numbered vocabularies), in which case every column is
 // read and updated in place.
+// The XCD (0..7) the calling wave runs on: bits 3:0 of hardware register XCC_ID (id 20).
+__device__ __forceinline__ int xcc_id() {
+  return (int)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1));
+}
+
 __device__ __forceinline__ Shadow resolve_hot_mode(Shadow sh) {
+  sh.xcc = xcc_id();
   if (sh.hot_total > 0) {
     int part = 0;
     for (int k = threadIdx.x & 63; k < kHotCountSlots; k += kWave) part += sh.hot_seen[k];
@@ -291,14 +303,35 @@ __device__ __forceinline__ int hot_index(const ColRef& ref, int combine) {
   return (combine == kHotCombining || ref.hot < kHotWordsExact) ? ref.hot : -1;
 }
 
-// `shadow` is the shadow buffer of ref's table (Shadow::a or Shadow::b).
+// The read copy of hot column `hot` of table `which` (0 = B, 1 = A) for this wave's XCD, or null.
+__device__ __forceinline__ float* read_copy(const Shadow& sh, int which, int hot, int d) {
+  float* const pub = which ? sh.pub_a : sh.pub_b;
+  return pub == nullptr ? nullptr : pub + ((int64_t)sh.xcc * kHotWords + hot) * d;
+}
+
+// Reads the column `ref` of table `which` (0 = B, 1 = A) as the mode of `sh` sees it.
+//   exact: the table column plus all its shadow copies.
+//   combining: the table column of a hot word receives the atomics of every fold, and reads of a
+//       line queue with the atomics to it, which made these few columns the critical path of the
+//       pass.  Readers therefore read a copy that no atomic ever touches: one per XCD (so that
+//       plain loads and stores through that XCD's L2 are coherent), filled from the table before
+//       the kernel for the hot ids the launch holds and rewritten by every fold done on the XCD
+//       with the value its atomic add to the table produced.
 template <int R>
-__device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const float* shadow,
-                                             int combine, int lane, int d) {
+__device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const Shadow& sh,
+                                             int which, int lane, int d) {
+  if (sh.combine == kHotCombining && ref.hot >= 0) {
+    const float* const pub = read_copy(sh, which, ref.hot, d);
+    if (pub != nullptr) {
+      load_col<R>(x, pub, lane, d);
+      return;
+    }
+  }
   load_col<R>(x, ref.col, lane, d);
-  if (combine == kHotExact && ref.hot >= 0 && ref.hot < kHotWordsExact) {
+  if (sh.combine == kHotExact && ref.hot >= 0 && ref.hot < kHotWordsExact) {
     // two copies per trip: enough loads in flight without inflating the register count of the
     // callers, which inline this many times
+    const float* const shadow = which ? sh.a : sh.b;
     const int copies = shadow_copies(ref.hot, 0);
 #pragma unroll 1
     for (int s = 0; s < copies; s += 2) {
@@ -311,17 +344,25 @@ __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, c
   }
 }
 
-// Moves what has piled up in a shadow copy into the table column it shadows.
+// Moves what has piled up in a shadow copy into the table column it shadows and, if the column
+// has a read copy on this XCD (`pub`, may be null), leaves the column's new value there.
 template <int R>
 __device__ __forceinline__ void fold_copy(float* __restrict__ copy, float* __restrict__ col,
-                                          int lane, int d) {
+                                          float* __restrict__ pub, int lane, int d) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int e = r * kWave + lane;
     if (r < R - 1 || e < d) {
       const float v =
           __hip_atomic_exchange(copy + e, 0.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (v != 0.0f) unsafeAtomicAdd(col + e, v);
+      if (v != 0.0f) {
+        if (pub != nullptr) {
+          const float before = unsafeAtomicAdd(col + e, v);
+          pub[e] = before + v;
+        } else {
+          unsafeAtomicAdd(col + e, v);
+        }
+      }
     }
   }
 }
@@ -358,7 +399,7 @@ __device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow&
   float* const copy = (which ? sh.a : sh.b) + ((int64_t)slot * kHotWords + hot) * d;
   atomic_add_col<R>(copy, x, lane, d);
   if (sh.combine == kHotCombining && ((ticket + 1u) & (kFoldEvery - 1)) == 0)
-    fold_copy<R>(copy, ref.col, lane, d);
+    fold_copy<R>(copy, ref.col, read_copy(sh, which, hot, d), lane, d);
 }
 
 // The same for callers on a rarely taken path: takes the ticket on the spot.

@@ -51,8 +51,25 @@ int get_hot_update_mode();
 void set_rare_update_mode(int mode);
 int get_rare_update_mode();
 size_t occurs_bytes();
-hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64_t nwg,
+// `ids` are the words read from table B (and counted), `ids2` those read from table A (null: the
+// same); A and B are the tables whose hot columns get read copies in the combining mode (null:
+// none, readers read the tables).
+hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
+                            int64_t n2, const float* A, const float* B, int d, int64_t nwg,
                             int waves_per_wg, Shadow* shadow);
+size_t read_copy_bytes();
+// Decides which words of a launch over `units` work units, `waves` of them in flight, are rare
+// enough for plain read-modify-write updates (Shadow::rare_max) and enqueues the count of the
+// words in the two id arrays (ids at or beyond idlimit are ignored).
+hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,
+                              int64_t nb, int idlimit, int64_t units, int64_t waves,
+                              Shadow* shadow);
+// For kernels that only read: no shadow copies anywhere.
+inline Shadow no_shadow() {
+  Shadow s{};
+  s.combine = kHotOff;
+  return s;
+}
 
 // Adds the shadow copies of the hot columns into A and B and zeroes them.
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);

@@ -149,7 +149,12 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
     if (lane < nwb) wbl = WB[unit * nwb + lane];
     if (wbl >= idlimit) wbl = -1;  // word2vecNegFilt: ids beyond the resident columns are skipped
     const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
-    const uint64_t rare_b = __ballot(wbl >= 0 && is_rare(shadow, wbl));
+    // a word that occurs twice in the group would have two plain updates in flight: not rare
+    bool lone_b = true;
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k)
+      if (k < nwb && k != lane && read_lane(wbl, k) == wbl) lone_b = false;
+    const uint64_t rare_b = __ballot(wbl >= 0 && lone_b && is_rare(shadow, wbl));
     // tickets for the writes to hot B columns at the end of the group, taken now
     const unsigned tkb = hot_ticket(shadow, 0, slot, (wbl >= 0 && wbl < kHotWords) ? wbl : -1);
 
@@ -165,7 +170,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
           if ((rare_b >> k) & 1)
             load_col_fresh<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
           else
-            load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow.b, shadow.combine, lane, d);
+            load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow, 0, lane, d);
         }
         zero_col<R>(dbb[k]);
       }
@@ -176,9 +181,14 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       if (jbase + lane < nwa) wal = WA[unit * nwa + jbase + lane];
       if (wal >= idlimit) wal = -1;
       const float sal = wal >= 0 ? scale_of(wal, vexp, smode) : 0.0f;
-      const uint64_t rare_a = __ballot(wal >= 0 && is_rare(shadow, wal));
-      const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
       const int jend = min(nwa - jbase, kWave);
+      bool lone_a = true;
+      if (shadow.rare_max > 0) {
+        for (int j = 0; j < jend; ++j)
+          if (j != lane && read_lane(wal, j) == wal) lone_a = false;
+      }
+      const uint64_t rare_a = __ballot(wal >= 0 && lone_a && is_rare(shadow, wal));
+      const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
         float a[CHA][R];
@@ -192,7 +202,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
               if ((rare_a >> (j0 + c)) & 1)
                 load_col_fresh<R>(a[c], A + (int64_t)wa[c] * d, lane, d);
               else
-                load_col_ref<R>(a[c], table_ref(A, wa[c], d), shadow.a, shadow.combine, lane, d);
+                load_col_ref<R>(a[c], table_ref(A, wa[c], d), shadow, 1, lane, d);
             }
           }
         }
@@ -257,17 +267,60 @@ __global__ void __launch_bounds__(kBlock) clear_occurs_kernel(int4* __restrict__
 // Counts how often each word occurs among the two id arrays of a launch, exactly up to rare_max
 // and saturating soon after: a slot that is already above rare_max is left alone, so the words that
 // occur hundreds of thousands of times do not queue that many atomics on one address.  Words that
-// may have shadow copies are never rare and are not counted.
+// may have shadow copies are never rare and are not counted.  Four ids per thread and trip, so
+// that the dependent id -> slot -> atomic chains of a thread overlap.
+__device__ __forceinline__ void count_occurrence(int w, int seen, int idlimit, int* occurs,
+                                                 int rare_max) {
+  if (w >= kHotWords && w < idlimit && seen <= rare_max)
+    __hip_atomic_fetch_add(occurs + (w & (kOccurSlots - 1)), 1, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ int peek_occurrence(int w, int idlimit, const int* occurs) {
+  // A plain load: an XCD sees the other XCDs' increments of a slot at the latest after its own
+  // next increment of it, so every XCD stops soon after the slot has passed rare_max.
+  return (w >= kHotWords && w < idlimit)
+             ? *const_cast<const volatile int*>(occurs + (w & (kOccurSlots - 1)))
+             : 0;
+}
+
+// `every` (a power of two): only every `every`-th run of 16 consecutive ids is looked at.  The id
+// arrays of the negative pass are in random order, so this is an unbiased sample, and the caller
+// scales its threshold accordingly.
 __global__ void __launch_bounds__(kBlock)
-count_occurs_kernel(const int* __restrict__ ids_a, int64_t na, const int* __restrict__ ids_b,
-                    int64_t nb, int idlimit, int* occurs, int rare_max) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < na + nb;
-       i += (int64_t)gridDim.x * kBlock) {
-    const int w = i < na ? ids_a[i] : ids_b[i - na];
-    if (w < kHotWords || w >= idlimit) continue;
-    int* const slot = occurs + (w & (kOccurSlots - 1));
-    if (__hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= rare_max)
-      __hip_atomic_fetch_add(slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+count_occurs_kernel(const int* __restrict__ ids, int64_t n, int every, int idlimit, int* occurs,
+                    int rare_max) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
+  const int64_t runs = n / 16;                        // whole runs of 16 ids
+  const int64_t kept = (runs + every - 1) / every;    // runs 0, every, 2 * every, ...
+  if (aligned) {
+    const int4* ids4 = reinterpret_cast<const int4*>(ids);
+    for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < kept * 4;
+         j += (int64_t)gridDim.x * kBlock) {
+      const int4 w = ids4[(j >> 2) * every * 4 + (j & 3)];
+      const int s0 = peek_occurrence(w.x, idlimit, occurs);
+      const int s1 = peek_occurrence(w.y, idlimit, occurs);
+      const int s2 = peek_occurrence(w.z, idlimit, occurs);
+      const int s3 = peek_occurrence(w.w, idlimit, occurs);
+      count_occurrence(w.x, s0, idlimit, occurs, rare_max);
+      count_occurrence(w.y, s1, idlimit, occurs, rare_max);
+      count_occurrence(w.z, s2, idlimit, occurs, rare_max);
+      count_occurrence(w.w, s3, idlimit, occurs, rare_max);
+    }
+  } else {
+    for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < kept * 16;
+         j += (int64_t)gridDim.x * kBlock) {
+      const int w = ids[(j >> 4) * every * 16 + (j & 15)];
+      count_occurrence(w, peek_occurrence(w, idlimit, occurs), idlimit, occurs, rare_max);
+    }
+  }
+  // the ids after the last whole run, when every id is looked at
+  if (every == 1) {
+    for (int64_t i = runs * 16 + (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * kBlock) {
+      const int w = ids[i];
+      count_occurrence(w, peek_occurrence(w, idlimit, occurs), idlimit, occurs, rare_max);
+    }
   }
 }
 
@@ -279,22 +332,33 @@ int get_rare_update_mode() { return g_rare_update_mode.load(); }
 // launch of `units` work units keeps `waves` of them in flight, so a word with n occurrences has
 // about n * waves / units updates in flight together; words for which that is below 1/16 are
 // updated without atomics.  Small launches get 0: everything stays atomic and nothing is counted.
+// The count is a scattered read-modify-write per id, which is what the device is slowest at, so for
+// thresholds that allow it only every 2nd, 4th or 8th run of ids is counted and the threshold
+// scaled down: the threshold is a soft one, and a word somewhat above it that slips through is as
+// harmless as one just below it.
 constexpr int kRareConcurrencyDen = 16;
 constexpr int kRareMaxCap = 64;
-static hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na,
-                                     const int* ids_b, int64_t nb, int idlimit, int64_t units,
-                                     int64_t waves, Shadow* shadow) {
+constexpr int kRareMinSampledMax = 3;   // the scaled threshold is kept at or above this
+hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,
+                              int64_t nb, int idlimit, int64_t units, int64_t waves,
+                              Shadow* shadow) {
   shadow->rare_max = 0;
   const int mode = g_rare_update_mode.load();
   if (mode == 0 || shadow->occurs == nullptr || waves <= 0) return hipSuccess;
   int64_t most = mode >= 2 ? mode : units / (kRareConcurrencyDen * waves);
   if (most > kRareMaxCap) most = kRareMaxCap;
   if (most < 1) return hipSuccess;
+  int every = 1;
+  while (every < 8 && most / (2 * every) >= kRareMinSampledMax) every *= 2;
+  const int sampled_max = (int)(most / every);
   hipLaunchKernelGGL(clear_occurs_kernel, dim3(256), dim3(kBlock), 0, stream,
                      reinterpret_cast<int4*>(shadow->occurs), kOccurSlots / 4);
-  hipLaunchKernelGGL(count_occurs_kernel, dim3(1024), dim3(kBlock), 0, stream, ids_a, na, ids_b, nb,
-                     idlimit, shadow->occurs, (int)most);
-  shadow->rare_max = (int)most;
+  hipLaunchKernelGGL(count_occurs_kernel, dim3(1024), dim3(kBlock), 0, stream, ids_a, na, every,
+                     idlimit, shadow->occurs, sampled_max);
+  if (nb > 0)
+    hipLaunchKernelGGL(count_occurs_kernel, dim3(1024), dim3(kBlock), 0, stream, ids_b, nb, every,
+                       idlimit, shadow->occurs, sampled_max);
+  shadow->rare_max = sampled_max;
   return hipGetLastError();
 }
 
@@ -337,7 +401,8 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   hipError_t err = split_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, ngroups,
                               kMinGroupsPerWg, kMinGroupsPerWgWide, &g);
   if (err != hipSuccess) return err;
-  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, g.nwg, kNegWaves, &shadow);
+  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa, A, B, d,
+                         g.nwg, kNegWaves, &shadow);
   if (err != hipSuccess) return err;
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;

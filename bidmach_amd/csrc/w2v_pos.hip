@@ -273,8 +273,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const ColRef r0 = tables.b(w0, d);
       const ColRef r1 = tables.b(w1, d);
       float x0[R], x1[R];
-      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.b, shadow.combine, lane, d);
-      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.b, shadow.combine, lane, d);
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow, 0, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow, 0, lane, d);
       if (lane == 0) {
         wt[c0] = r0.flags != 0 ? w0 : -1;
         ft[c0] = r0.flags;
@@ -299,8 +299,8 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
       const ColRef r0 = tables.a(w0, d);
       const ColRef r1 = tables.a(w1, d);
       float x0[R], x1[R];
-      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow.a, shadow.combine, lane, d);
-      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow.a, shadow.combine, lane, d);
+      if (r0.flags != 0) load_col_ref<R>(x0, r0, shadow, 1, lane, d);
+      if (r1.flags != 0) load_col_ref<R>(x1, r1, shadow, 1, lane, d);
       if (r0.flags != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) a_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
@@ -380,7 +380,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
         const ColRef rb = tables.b(wb, d);
         if (rb.flags == 0 || !tables.trained(fi, rb.flags)) continue;
         float b[R];
-        load_col_ref<R>(b, rb, shadow.b, shadow.combine, lane, d);
+        load_col_ref<R>(b, rb, shadow, 0, lane, d);
         const float s = wave_sum(dot_partial<R>(a, b));
         const float g = lrate * (1.0f - sat_sigmoid(s));
         axpy<R>(daa, ascale * g, b);
@@ -454,47 +454,99 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
   }
 }
 
-// Counts the word ids below kHotWords: block b leaves its share in out[b] (kHotCountSlots blocks,
-// every slot is written on every launch, so nothing needs clearing and no atomics queue up).
+// Counts the word ids below kHotWords among `ids`: block b leaves its share in out[b]
+// (kHotCountSlots blocks, every slot is written on every launch, so nothing needs clearing and no
+// atomics queue up).  It also leaves, in mask[b] and mask[kHotCountSlots + b], bit masks of the hot
+// ids it saw in `ids` (the words read from table B) and in `ids2` (those read from table A; null:
+// the same as `ids`).
 __global__ void __launch_bounds__(kBlock)
-count_hot_kernel(const int* __restrict__ ids, int64_t n, int* __restrict__ out) {
-  __shared__ int s_part[kWavesPerBlock];
-  int local = 0;
-  const int64_t n4 = n / 4;
-  const int4* ids4 = reinterpret_cast<const int4*>(ids);   // device allocations are 16-byte aligned
-  const bool aligned = (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
+count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
+                 int* __restrict__ out, int* __restrict__ mask) {
+  __shared__ int s_part[kWavesPerBlock], s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
+  int local = 0, seen = 0, seen2 = 0;
   auto hot = [](int w) { return (w >= 0 && w < kHotWords) ? 1 : 0; };
-  if (aligned) {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4;
-         i += (int64_t)gridDim.x * kBlock) {
-      const int4 v = ids4[i];
-      local += hot(v.x) + hot(v.y) + hot(v.z) + hot(v.w);
+  auto bit = [](int w) { return (w >= 0 && w < kHotWords) ? (1 << w) : 0; };
+  auto scan = [&](const int* p, int64_t len, int& count, int& bits) {
+    const int64_t len4 = len / 4;
+    const int4* p4 = reinterpret_cast<const int4*>(p);   // device allocations are 16-byte aligned
+    const bool aligned = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+    if (aligned) {
+      for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < len4;
+           i += (int64_t)gridDim.x * kBlock) {
+        const int4 v = p4[i];
+        count += hot(v.x) + hot(v.y) + hot(v.z) + hot(v.w);
+        bits |= bit(v.x) | bit(v.y) | bit(v.z) | bit(v.w);
+      }
     }
-    for (int64_t i = n4 * 4 + (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
-         i += (int64_t)gridDim.x * kBlock)
-      local += hot(ids[i]);
+    for (int64_t i = (aligned ? len4 * 4 : 0) + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+         i < len; i += (int64_t)gridDim.x * kBlock) {
+      count += hot(p[i]);
+      bits |= bit(p[i]);
+    }
+  };
+  scan(ids, n, local, seen);
+  if (ids2 != nullptr) {
+    int unused = 0;
+    scan(ids2, n2, unused, seen2);
   } else {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
-         i += (int64_t)gridDim.x * kBlock)
-      local += hot(ids[i]);
+    seen2 = seen;
   }
 #pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) local += __shfl_xor(local, m, kWave);
-  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
+  for (int m = 32; m >= 1; m >>= 1) {
+    local += __shfl_xor(local, m, kWave);
+    seen |= __shfl_xor(seen, m, kWave);
+    seen2 |= __shfl_xor(seen2, m, kWave);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_part[threadIdx.x >> 6] = local;
+    s_mask[threadIdx.x >> 6] = seen;
+    s_mask2[threadIdx.x >> 6] = seen2;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
-    int total = 0;
+    int total = 0, m1 = 0, m2 = 0;
 #pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      total += s_part[w];
+      m1 |= s_mask[w];
+      m2 |= s_mask2[w];
+    }
     out[blockIdx.x] = total;
+    mask[blockIdx.x] = m1;
+    mask[kHotCountSlots + blockIdx.x] = m2;
+  }
+}
+
+// Fills the per-XCD read copies of the hot columns the launch holds (block (w, t): word w of
+// table t, 0 = B, 1 = A) from the tables.  Words the launch does not hold are skipped, so the
+// vocabulary may be smaller than kHotWords.
+__global__ void __launch_bounds__(kBlock)
+publish_kernel(const float* __restrict__ A, const float* __restrict__ B, Shadow shadow, int d) {
+  __shared__ int s_mask;
+  const int w = blockIdx.x, which = blockIdx.y;
+  if (threadIdx.x == 0) s_mask = 0;
+  __syncthreads();
+  int m = 0;
+  for (int k = threadIdx.x; k < kHotCountSlots; k += kBlock)
+    m |= shadow.hot_mask[which * kHotCountSlots + k];
+  if (m != 0) atomicOr(&s_mask, m);
+  __syncthreads();
+  if (((s_mask >> w) & 1) == 0) return;
+  const float* const col = (which ? A : B) + (int64_t)w * d;
+  float* const pub = which ? shadow.pub_a : shadow.pub_b;
+  for (int e = threadIdx.x; e < d; e += kBlock) {
+    const float v = col[e];
+#pragma unroll
+    for (int x = 0; x < kXcds; ++x) pub[((int64_t)x * kHotWords + w) * d + e] = v;
   }
 }
 
 size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
 size_t shadow_counter_bytes() {
   return (size_t)2 * kShadows * kHotWords * kCounterStride * sizeof(unsigned) +
-         (size_t)kHotCountSlots * sizeof(int);
+         (size_t)3 * kHotCountSlots * sizeof(int);   // hot-word counts and the two id masks
 }
+size_t read_copy_bytes() { return (size_t)kXcds * kHotWords * kMaxRounds * kWave * sizeof(float); }
 
 size_t occurs_bytes() { return (size_t)kOccurSlots * sizeof(int); }
 
@@ -517,21 +569,28 @@ int get_hot_update_mode() { return g_hot_update_mode.load(); }
 // invisible to each other anyway; with the Zipf share of the top word that is several hundred
 // invisible updates of that word per 2048 waves.  Below that size the exact mode is used.
 constexpr int64_t kCombineMinWaves = 2048;
-hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, int64_t nwg,
+hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
+                            int64_t n2, const float* A, const float* B, int d, int64_t nwg,
                             int waves_per_wg, Shadow* shadow) {
   const int mode = g_hot_update_mode.load();
   shadow->hot_total = 0;
-  if (mode == kHotExact || mode == kHotCombining || mode == kHotOff) {
+  if (A == nullptr || B == nullptr) shadow->pub_a = shadow->pub_b = nullptr;
+  const bool forced = mode == kHotExact || mode == kHotCombining || mode == kHotOff;
+  if (forced)
     shadow->combine = mode;
-    return hipSuccess;
-  }
-  shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
-  if (n <= 0) return hipSuccess;
+  else
+    shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
+  if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
+  if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
-  // read the count from memory, the host does not wait for it).
-  hipLaunchKernelGGL(count_hot_kernel, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids, n,
-                     shadow->hot_seen);
-  shadow->hot_total = n;
+  // read the count from memory, the host does not wait for it).  The same pass notes which hot
+  // ids occur at all, for the read copies.
+  hipLaunchKernelGGL(count_hot_kernel, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids, n, ids2,
+                     n2, shadow->hot_seen, shadow->hot_mask);
+  if (!forced) shadow->hot_total = n;
+  if (shadow->pub_a != nullptr)
+    hipLaunchKernelGGL(publish_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, *shadow,
+                       d);
   return hipGetLastError();
 }
 
@@ -679,7 +738,9 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   err = split_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, ntiles, kMinTilesPerWg,
                    kMinTilesPerWgWide, &g);
   if (err != hipSuccess) return err;
-  err = prepare_hot_mode(stream, W, ncols, g.nwg, kTileWaves, &shadow);
+  // the read copies serve the single-table model only
+  err = prepare_hot_mode(stream, W, ncols, nullptr, 0, Tables::kSliced ? nullptr : fold_a,
+                         Tables::kSliced ? nullptr : fold_b, d, g.nwg, kTileWaves, &shadow);
   if (err != hipSuccess) return err;
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;

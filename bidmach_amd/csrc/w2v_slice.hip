@@ -61,7 +61,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
     const int jlo = max(LB[i], -i);
     const int jhi = min(UB[i], ncols - 1 - i);
     float a[R];
-    load_col_ref<R>(a, pa, shadow.a, TRAIN ? shadow.combine : kHotOff, lane, d);
+    load_col_ref<R>(a, pa, shadow, 1, lane, d);
     float daa[R];
     zero_col<R>(daa);
     const float ascale = TRAIN ? scale_of(wi, vexp, smode) : 1.0f;
@@ -97,7 +97,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
         for (int c = 0; c < CH; ++c) {
           if (c < n) {
             rb[c] = read_lane_ref(pb, src[c]);
-            load_col_ref<R>(b[c], rb[c], shadow.b, TRAIN ? shadow.combine : kHotOff, lane, d);
+            load_col_ref<R>(b[c], rb[c], shadow, 0, lane, d);
           }
         }
         float pre = 0.0f;
@@ -154,6 +154,15 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     if (lane < nwb) wbl = WB[unit * nwb + lane];
     const ColRef pbl = tables.b(wbl, d);
     const float sbl = (TRAIN && pbl.flags != 0) ? scale_of(wbl, vexp, smode) : 0.0f;
+    // words updated without atomics: rare in this launch, written, and only once in the group
+    uint64_t rare_b = 0;
+    if (TRAIN && shadow.rare_max > 0) {
+      bool lone = true;
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k)
+        if (k < nwb && k != lane && read_lane(wbl, k) == wbl) lone = false;
+      rare_b = __ballot(lone && pbl.hot < 0 && tables.written(pbl.flags) && is_rare(shadow, wbl));
+    }
     // tickets for the writes to hot B columns at the end of the group, taken now
     const unsigned tkb =
         (TRAIN && tables.written(pbl.flags)) ? hot_ticket(shadow, 0, slot, pbl.hot) : 0u;
@@ -169,8 +178,12 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
       if (k < nwb) {
         rb[k] = read_lane_ref(pbl, k);
         fb[k] = rb[k].flags;
-        if (fb[k] != 0)
-          load_col_ref<R>(b[k], rb[k], shadow.b, TRAIN ? shadow.combine : kHotOff, lane, d);
+        if (fb[k] != 0) {
+          if ((rare_b >> k) & 1)
+            load_col_fresh<R>(b[k], rb[k].col, lane, d);
+          else
+            load_col_ref<R>(b[k], rb[k], shadow, 0, lane, d);
+        }
         zero_col<R>(dbb[k]);
       }
     }
@@ -183,6 +196,13 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
       const unsigned tka =
           (TRAIN && tables.written(pal.flags)) ? hot_ticket(shadow, 1, slot, pal.hot) : 0u;
       const int jend = min(nwa - jbase, kWave);
+      uint64_t rare_a = 0;
+      if (TRAIN && shadow.rare_max > 0) {
+        bool lone = true;
+        for (int j = 0; j < jend; ++j)
+          if (j != lane && read_lane(wal, j) == wal) lone = false;
+        rare_a = __ballot(lone && pal.hot < 0 && tables.written(pal.flags) && is_rare(shadow, wal));
+      }
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
         float a[CHA][R];
@@ -195,8 +215,12 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
           if (j0 + c < jend) {
             ra[c] = read_lane_ref(pal, j0 + c);
             fa[c] = ra[c].flags;
-            if (fa[c] != 0)
-              load_col_ref<R>(a[c], ra[c], shadow.a, TRAIN ? shadow.combine : kHotOff, lane, d);
+            if (fa[c] != 0) {
+              if ((rare_a >> (j0 + c)) & 1)
+                load_col_fresh<R>(a[c], ra[c].col, lane, d);
+              else
+                load_col_ref<R>(a[c], ra[c], shadow, 1, lane, d);
+            }
           }
         }
         float pre = 0.0f;
@@ -232,7 +256,9 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
                   axpy<R>(daa, as * g, b[k]);
                 }
               }
-              if (tables.written(fa[c]))
+              if ((rare_a >> (j0 + c)) & 1)
+                store_sum_col<R>(ra[c].col, a[c], daa, lane, d);
+              else if (tables.written(fa[c]))
                 scatter_add_ref<R>(ra[c], shadow, 1, slot, daa, lane, d, read_lane(tka, j0 + c));
             }
           }
@@ -245,7 +271,9 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     if (TRAIN) {
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
-        if (fb[k] != 0 && tables.written(fb[k]))
+        if ((rare_b >> k) & 1)
+          store_sum_col<R>(rb[k].col, b[k], dbb[k], lane, d);
+        else if (fb[k] != 0 && tables.written(fb[k]))
           scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d, read_lane(tkb, k));
       }
     }
@@ -292,7 +320,8 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ncols, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   if (TRAIN) {
-    err = prepare_hot_mode(stream, W, ncols, nwg, kWavesPerBlock, &shadow);
+    err = prepare_hot_mode(stream, W, ncols, nullptr, 0, nullptr, nullptr, d, nwg,
+                           kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
@@ -311,7 +340,11 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ngroups, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   if (TRAIN) {
-    err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nwg, kWavesPerBlock, &shadow);
+    err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nullptr, 0, nullptr, nullptr, d,
+                           nwg, kWavesPerBlock, &shadow);
+    if (err != hipSuccess) return err;
+    err = prepare_rare_words(stream, WA, (int64_t)ngroups * nwa, WB, (int64_t)ngroups * nwb,
+                             0x7fffffff, ngroups, nwg * kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
@@ -378,7 +411,7 @@ hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const
   int64_t nparts = 0;
 #define CALL(R)                                                                                   \
   err = launch_slice_pos_r<R, false>(stream, nrows, ncols, W, LB, UB, m, 0.0f, 0.0f, floorv,      \
-                                     partials, &nparts, Shadow{});                                \
+                                     partials, &nparts, no_shadow());                                \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
@@ -394,7 +427,7 @@ hipError_t launch_slice_eval_neg(hipStream_t stream, int nrows, int ncols, int n
   int64_t nparts = 0;
 #define CALL(R)                                                                                   \
   err = launch_slice_neg_r<R, false>(stream, nrows, ncols, nwa, nwb, WA, WB, m, 0.0f, 0.0f,       \
-                                     floorv, partials, &nparts, Shadow{});                        \
+                                     floorv, partials, &nparts, no_shadow());                        \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL

@@ -8,6 +8,7 @@ import pytest
 
 from bidmach_amd import corpus
 from tests import test_gpu_parity as parity
+from tests import test_gpu_slice as sliced
 
 pytestmark = pytest.mark.gpu
 
@@ -34,6 +35,15 @@ def test_collision_free_updates_match_oracle(gpu, oracle, rare_mode):
         parity.test_neg_update_matches_oracle(gpu, oracle, vexp, 1280, 5, 5, 30)
         parity.test_neg_update_matches_oracle(gpu, oracle, vexp, 40, 70, 3, 40)
     parity.test_neg_filt_matches_oracle(gpu, oracle, 100, 10, 5)
+
+
+def test_sliced_model_matches_oracle(gpu, oracle, rare_mode):
+    """Collision-free groups against a sliced, multi-part model: columns that are not written
+    (read-only head words, words of other workers) must stay bit-identical too."""
+    for slicing in sliced.SLICINGS:
+        sliced.test_neg_slice_matches_oracle(gpu, oracle, *slicing, 100, 5, 5, 0.0)
+        sliced.test_neg_slice_matches_oracle(gpu, oracle, *slicing, 130, 3, 8, 0.5)
+        sliced.test_neg_slice_matches_oracle(gpu, oracle, *slicing, 64, 70, 2, 0.0)
 
 
 def test_plain_path_is_bit_identical_to_atomics_without_collisions(gpu, rare_mode):
