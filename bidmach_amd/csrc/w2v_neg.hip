@@ -338,7 +338,7 @@ int get_rare_update_mode() { return g_rare_update_mode.load(); }
 // harmless as one just below it.
 constexpr int kRareConcurrencyDen = 16;
 constexpr int kRareMaxCap = 64;
-constexpr int kRareMinSampledMax = 3;   // the scaled threshold is kept at or above this
+constexpr int kRareMinSampledMax = 2;   // the scaled threshold is kept at or above this
 hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,
                               int64_t nb, int idlimit, int64_t units, int64_t waves,
                               Shadow* shadow) {
