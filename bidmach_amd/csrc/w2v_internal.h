@@ -57,6 +57,10 @@ size_t occurs_bytes();
 hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
                             int64_t n2, const float* A, const float* B, int d, int64_t nwg,
                             int waves_per_wg, Shadow* shadow);
+// The same for a sliced model, whose shadowed columns are the first columns of part 0.
+hipError_t prepare_hot_mode_sliced(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
+                                   int64_t n2, const SliceMap& m, int d, int64_t nwg,
+                                   int waves_per_wg, Shadow* shadow);
 size_t read_copy_bytes();
 // Decides which words of a launch over `units` work units, `waves` of them in flight, are rare
 // enough for plain read-modify-write updates (Shadow::rare_max) and enqueues the count of the

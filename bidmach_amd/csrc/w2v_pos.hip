@@ -458,15 +458,23 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
 // (kHotCountSlots blocks, every slot is written on every launch, so nothing needs clearing and no
 // atomics queue up).  It also leaves, in mask[b] and mask[kHotCountSlots + b], bit masks of the hot
 // ids it saw in `ids` (the words read from table B) and in `ids2` (those read from table A; null:
-// the same as `ids`).
+// the same as `ids`); there a word counts under the index of its shadow copies (ColRef::hot), which
+// for a sliced model is its packed column and not its id.
+template <class Tables>
 __global__ void __launch_bounds__(kBlock)
 count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
-                 int* __restrict__ out, int* __restrict__ mask) {
+                 Tables tables, int* __restrict__ out, int* __restrict__ mask) {
   __shared__ int s_part[kWavesPerBlock], s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
   int local = 0, seen = 0, seen2 = 0;
   auto hot = [](int w) { return (w >= 0 && w < kHotWords) ? 1 : 0; };
-  auto bit = [](int w) { return (w >= 0 && w < kHotWords) ? (1 << w) : 0; };
-  auto scan = [&](const int* p, int64_t len, int& count, int& bits) {
+  auto scan = [&](const int* p, int64_t len, int& count, int& bits, bool of_a) {
+    auto bit = [&](int w) {
+      if (Tables::kSliced) {
+        const int h = w >= 0 ? (of_a ? tables.a(w, 0).hot : tables.b(w, 0).hot) : -1;
+        return h >= 0 ? (1 << h) : 0;
+      }
+      return (w >= 0 && w < kHotWords) ? (1 << w) : 0;
+    };
     const int64_t len4 = len / 4;
     const int4* p4 = reinterpret_cast<const int4*>(p);   // device allocations are 16-byte aligned
     const bool aligned = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
@@ -484,10 +492,10 @@ count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__
       bits |= bit(p[i]);
     }
   };
-  scan(ids, n, local, seen);
-  if (ids2 != nullptr) {
+  scan(ids, n, local, seen, false);
+  if (ids2 != nullptr || Tables::kSliced) {
     int unused = 0;
-    scan(ids2, n2, unused, seen2);
+    scan(ids2 != nullptr ? ids2 : ids, ids2 != nullptr ? n2 : n, unused, seen2, true);
   } else {
     seen2 = seen;
   }
@@ -569,9 +577,11 @@ int get_hot_update_mode() { return g_hot_update_mode.load(); }
 // invisible to each other anyway; with the Zipf share of the top word that is several hundred
 // invisible updates of that word per 2048 waves.  Below that size the exact mode is used.
 constexpr int64_t kCombineMinWaves = 2048;
-hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
-                            int64_t n2, const float* A, const float* B, int d, int64_t nwg,
-                            int waves_per_wg, Shadow* shadow) {
+template <class Tables>
+static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64_t n,
+                                       const int* ids2, int64_t n2, const Tables& tables,
+                                       const float* A, const float* B, int d, int64_t nwg,
+                                       int waves_per_wg, Shadow* shadow) {
   const int mode = g_hot_update_mode.load();
   shadow->hot_total = 0;
   if (A == nullptr || B == nullptr) shadow->pub_a = shadow->pub_b = nullptr;
@@ -585,13 +595,28 @@ hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
   // read the count from memory, the host does not wait for it).  The same pass notes which hot
   // ids occur at all, for the read copies.
-  hipLaunchKernelGGL(count_hot_kernel, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids, n, ids2,
-                     n2, shadow->hot_seen, shadow->hot_mask);
+  hipLaunchKernelGGL(count_hot_kernel<Tables>, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids,
+                     n, ids2, n2, tables, shadow->hot_seen, shadow->hot_mask);
   if (!forced) shadow->hot_total = n;
   if (shadow->pub_a != nullptr)
     hipLaunchKernelGGL(publish_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, *shadow,
                        d);
   return hipGetLastError();
+}
+
+hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
+                            int64_t n2, const float* A, const float* B, int d, int64_t nwg,
+                            int waves_per_wg, Shadow* shadow) {
+  return prepare_hot_mode_for(stream, ids, n, ids2, n2, PlainTables{nullptr, nullptr}, A, B, d, nwg,
+                              waves_per_wg, shadow);
+}
+
+hipError_t prepare_hot_mode_sliced(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
+                                   int64_t n2, const SliceMap& m, int d, int64_t nwg,
+                                   int waves_per_wg, Shadow* shadow) {
+  // the shadowed columns are the first columns of part 0
+  return prepare_hot_mode_for(stream, ids, n, ids2, n2, SlicedTables{m}, m.mats[1], m.mats[0], d,
+                              nwg, waves_per_wg, shadow);
 }
 
 hipError_t persistent_grid(const void* kernel, int threads, size_t lds_bytes, int64_t units,
@@ -738,9 +763,12 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   err = split_grid(reinterpret_cast<const void*>(kern), kTileThreads, lds, ntiles, kMinTilesPerWg,
                    kMinTilesPerWgWide, &g);
   if (err != hipSuccess) return err;
-  // the read copies serve the single-table model only
-  err = prepare_hot_mode(stream, W, ncols, nullptr, 0, Tables::kSliced ? nullptr : fold_a,
-                         Tables::kSliced ? nullptr : fold_b, d, g.nwg, kTileWaves, &shadow);
+  if constexpr (Tables::kSliced)
+    err = prepare_hot_mode_sliced(stream, W, ncols, nullptr, 0, tables.m, d, g.nwg, kTileWaves,
+                                  &shadow);
+  else
+    err = prepare_hot_mode(stream, W, ncols, nullptr, 0, fold_a, fold_b, d, g.nwg, kTileWaves,
+                           &shadow);
   if (err != hipSuccess) return err;
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;

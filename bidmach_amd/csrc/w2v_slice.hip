@@ -320,8 +320,7 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ncols, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   if (TRAIN) {
-    err = prepare_hot_mode(stream, W, ncols, nullptr, 0, nullptr, nullptr, d, nwg,
-                           kWavesPerBlock, &shadow);
+    err = prepare_hot_mode_sliced(stream, W, ncols, nullptr, 0, m, d, nwg, kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
@@ -340,8 +339,8 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
   hipError_t err = slice_grid(reinterpret_cast<const void*>(kern), ngroups, &nwg, &per_wg);
   if (err != hipSuccess) return err;
   if (TRAIN) {
-    err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, nullptr, 0, nullptr, nullptr, d,
-                           nwg, kWavesPerBlock, &shadow);
+    err = prepare_hot_mode_sliced(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa, m,
+                                  d, nwg, kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
     err = prepare_rare_words(stream, WA, (int64_t)ngroups * nwa, WB, (int64_t)ngroups * nwb,
                              0x7fffffff, ngroups, nwg * kWavesPerBlock, &shadow);
