@@ -84,12 +84,14 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   out->occurs = reinterpret_cast<int*>(reinterpret_cast<char*>(out->count) +
                                        w2v::shadow_counter_bytes());
   out->rare_max = 0;
-  out->hot_mask = out->hot_seen + w2v::kHotCountSlots;
+  out->hot_mask = out->hot_seen + 4 * w2v::kHotCountSlots;
   out->pub_a = reinterpret_cast<float*>(reinterpret_cast<char*>(out->occurs) + w2v::occurs_bytes());
   out->pub_b = out->pub_a + w2v::read_copy_bytes() / sizeof(float);
   out->xcc = 0;
   out->hot_total = 0;
+  out->hot_total_a = 0;
   out->combine = 0;
+  out->combine_a = 0;
   return hipSuccess;
 }
 

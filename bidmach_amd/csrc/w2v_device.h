@@ -214,6 +214,7 @@ constexpr int kCounterStride = 32;  // one write counter per 128-byte line
 
 enum HotMode : int { kHotExact = 0, kHotCombining = 1, kHotOff = 2 };
 constexpr int kHotShareDen = 16;  // shadows are used if >= 1/16 of a launch's ids are hot words
+constexpr int kHotZeroShareDen = 48;  // or if >= 1/48 of them are id 0
 constexpr int kHotCountSlots = 256;  // blocks of the counting kernel, one partial count each
 
 struct Shadow {
@@ -221,10 +222,15 @@ struct Shadow {
   float* b;         // same for table B
   unsigned* count;  // [2][kShadows][kHotWords][kCounterStride] write counters (B then A); they
                     // only ever count up, so they need no clearing between calls
-  int* hot_seen;        // kHotCountSlots partial counts: how many of the launch's `hot_total` word
-  long long hot_total;  // ids are below kHotWords, counted on the device before the launch;
-                        // hot_total == 0: not counted
-  int combine;          // kHotExact or kHotCombining (kHotOff once resolved in a kernel)
+  // Counted on the device before the launch, kHotCountSlots partial counts each: how many of the
+  // hot_total word ids read from table B are below kHotWords, how many are 0, and the same two
+  // for the hot_total_a ids read from table A (0: table A follows table B).  hot_total == 0: not
+  // counted, the modes below stand.
+  int* hot_seen;
+  long long hot_total;
+  long long hot_total_a;
+  int combine;    // table B: kHotExact or kHotCombining (kHotOff once resolved in a kernel)
+  int combine_a;  // table A
   // Rare words.  The float-atomic units are what bounds the update passes, and most of their work
   // is spent on columns that are touched a handful of times per launch, where two updates of the
   // same column are practically never in flight together.  occurs[w & (kOccurSlots - 1)] holds how
@@ -258,23 +264,48 @@ __device__ __forceinline__ int xcc_id() {
   return (int)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1));
 }
 
+// Sum over the kHotCountSlots partial counts at `part`, the same value in every lane.
+__device__ __forceinline__ long long sum_hot_counts(const int* part) {
+  int t = 0;
+  for (int k = threadIdx.x & 63; k < kHotCountSlots; k += kWave) t += part[k];
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) t += __shfl_xor(t, m, kWave);
+  return __builtin_amdgcn_readfirstlane(t);
+}
+
+// Whether `total` word ids with `low` of them below kHotWords and `zero` of them equal to 0 are
+// worth shadow copies: the 16 lowest ids are a sixteenth of all, or id 0 alone is a 48th (its
+// atomics retire one after the other, and at 5 ids per group a 48th of them already lasts about
+// half as long as the whole pass).
+__device__ __forceinline__ bool ids_are_hot(long long low, long long zero, long long total) {
+  return low * kHotShareDen >= total || zero * kHotZeroShareDen >= total;
+}
+
 __device__ __forceinline__ Shadow resolve_hot_mode(Shadow sh) {
   sh.xcc = xcc_id();
   if (sh.hot_total > 0) {
-    int part = 0;
-    for (int k = threadIdx.x & 63; k < kHotCountSlots; k += kWave) part += sh.hot_seen[k];
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) part += __shfl_xor(part, m, kWave);
-    const long long seen = __builtin_amdgcn_readfirstlane(part);
-    if (seen * kHotShareDen < sh.hot_total) sh.combine = kHotOff;
+    const bool hot_b = ids_are_hot(sum_hot_counts(sh.hot_seen),
+                                   sum_hot_counts(sh.hot_seen + kHotCountSlots), sh.hot_total);
+    bool hot_a = hot_b;
+    if (sh.hot_total_a > 0)
+      hot_a = ids_are_hot(sum_hot_counts(sh.hot_seen + 2 * kHotCountSlots),
+                          sum_hot_counts(sh.hot_seen + 3 * kHotCountSlots), sh.hot_total_a);
+    if (!hot_b) sh.combine = kHotOff;
+    if (!hot_a) sh.combine_a = kHotOff;
   }
   return sh;
+}
+
+// The mode of table `which` (0 = B, 1 = A).
+__device__ __forceinline__ int hot_mode_of(const Shadow& sh, int which) {
+  return which ? sh.combine_a : sh.combine;
 }
 
 // True if the launch counted its hot words and found too few: such a launch has no column that a
 // large share of the units in flight would update, so it may spread over the whole device.
 __device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow& resolved) {
-  return asked.hot_total > 0 && asked.combine != kHotOff && resolved.combine == kHotOff;
+  return asked.hot_total > 0 && asked.combine != kHotOff && resolved.combine == kHotOff &&
+         resolved.combine_a == kHotOff;
 }
 
 __device__ __forceinline__ int shadow_copies(int w, int combine) {
@@ -320,7 +351,8 @@ __device__ __forceinline__ float* read_copy(const Shadow& sh, int which, int hot
 template <int R>
 __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, const Shadow& sh,
                                              int which, int lane, int d) {
-  if (sh.combine == kHotCombining && ref.hot >= 0) {
+  const int mode = hot_mode_of(sh, which);
+  if (mode == kHotCombining && ref.hot >= 0) {
     const float* const pub = read_copy(sh, which, ref.hot, d);
     if (pub != nullptr) {
       load_col<R>(x, pub, lane, d);
@@ -328,7 +360,7 @@ __device__ __forceinline__ void load_col_ref(float (&x)[R], const ColRef& ref, c
     }
   }
   load_col<R>(x, ref.col, lane, d);
-  if (sh.combine == kHotExact && ref.hot >= 0 && ref.hot < kHotWordsExact) {
+  if (mode == kHotExact && ref.hot >= 0 && ref.hot < kHotWordsExact) {
     // two copies per trip: enough loads in flight without inflating the register count of the
     // callers, which inline this many times
     const float* const shadow = which ? sh.a : sh.b;
@@ -372,7 +404,7 @@ __device__ __forceinline__ void fold_copy(float* __restrict__ copy, float* __res
 // The returning atomic takes a few microseconds, so callers take the ticket well before the write
 // it belongs to.  0 when the write will not go to a combining shadow copy.
 __device__ __forceinline__ unsigned hot_ticket(const Shadow& sh, int which, int wg, int hot) {
-  if (sh.combine != kHotCombining || hot < 0) return 0u;
+  if (hot_mode_of(sh, which) != kHotCombining || hot < 0) return 0u;
   const int slot = wg & (shadow_copies(hot, kHotCombining) - 1);
   unsigned* const counter =
       sh.count + (((int64_t)which * kShadows + slot) * kHotWords + hot) * kCounterStride;
@@ -390,15 +422,16 @@ template <int R>
 __device__ __forceinline__ void scatter_add_ref(const ColRef& ref, const Shadow& sh, int which,
                                                 int wg, const float (&x)[R], int lane, int d,
                                                 unsigned ticket) {
-  const int hot = hot_index(ref, sh.combine);
+  const int mode = hot_mode_of(sh, which);
+  const int hot = hot_index(ref, mode);
   if (hot < 0) {
     atomic_add_col<R>(ref.col, x, lane, d);
     return;
   }
-  const int slot = wg & (shadow_copies(hot, sh.combine) - 1);
+  const int slot = wg & (shadow_copies(hot, mode) - 1);
   float* const copy = (which ? sh.a : sh.b) + ((int64_t)slot * kHotWords + hot) * d;
   atomic_add_col<R>(copy, x, lane, d);
-  if (sh.combine == kHotCombining && ((ticket + 1u) & (kFoldEvery - 1)) == 0)
+  if (mode == kHotCombining && ((ticket + 1u) & (kFoldEvery - 1)) == 0)
     fold_copy<R>(copy, ref.col, read_copy(sh, which, hot, d), lane, d);
 }
 

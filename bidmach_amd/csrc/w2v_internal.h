@@ -72,6 +72,7 @@ hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, 
 inline Shadow no_shadow() {
   Shadow s{};
   s.combine = kHotOff;
+  s.combine_a = kHotOff;
   return s;
 }
 

@@ -454,9 +454,9 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
   }
 }
 
-// Counts the word ids below kHotWords among `ids`: block b leaves its share in out[b]
-// (kHotCountSlots blocks, every slot is written on every launch, so nothing needs clearing and no
-// atomics queue up).  It also leaves, in mask[b] and mask[kHotCountSlots + b], bit masks of the hot
+// Counts the word ids below kHotWords, and those equal to 0, among `ids` and among `ids2`: block b
+// leaves its four shares in out[k * kHotCountSlots + b] (kHotCountSlots blocks, every slot is
+// written on every launch, so nothing needs clearing and no atomics queue up).  It also leaves, in mask[b] and mask[kHotCountSlots + b], bit masks of the hot
 // ids it saw in `ids` (the words read from table B) and in `ids2` (those read from table A; null:
 // the same as `ids`); there a word counts under the index of its shadow copies (ColRef::hot), which
 // for a sliced model is its packed column and not its id.
@@ -464,9 +464,11 @@ template <class Tables>
 __global__ void __launch_bounds__(kBlock)
 count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
                  Tables tables, int* __restrict__ out, int* __restrict__ mask) {
-  __shared__ int s_part[kWavesPerBlock], s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
-  int local = 0, seen = 0, seen2 = 0;
-  auto hot = [](int w) { return (w >= 0 && w < kHotWords) ? 1 : 0; };
+  __shared__ int s_part[4][kWavesPerBlock], s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
+  int local = 0, zero = 0, local2 = 0, zero2 = 0, seen = 0, seen2 = 0;
+  // low 16 bits: 1 for an id below kHotWords; high 16 bits: 1 for id 0 (a thread sees far fewer
+  // than 65536 ids)
+  auto hot = [](int w) { return ((w >= 0 && w < kHotWords) ? 1 : 0) + (w == 0 ? 0x10000 : 0); };
   auto scan = [&](const int* p, int64_t len, int& count, int& bits, bool of_a) {
     auto bit = [&](int w) {
       if (Tables::kSliced) {
@@ -494,32 +496,45 @@ count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__
   };
   scan(ids, n, local, seen, false);
   if (ids2 != nullptr || Tables::kSliced) {
-    int unused = 0;
-    scan(ids2 != nullptr ? ids2 : ids, ids2 != nullptr ? n2 : n, unused, seen2, true);
+    scan(ids2 != nullptr ? ids2 : ids, ids2 != nullptr ? n2 : n, local2, seen2, true);
   } else {
     seen2 = seen;
   }
+  zero = local >> 16;
+  local &= 0xffff;
+  zero2 = local2 >> 16;
+  local2 &= 0xffff;
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) {
     local += __shfl_xor(local, m, kWave);
+    zero += __shfl_xor(zero, m, kWave);
+    local2 += __shfl_xor(local2, m, kWave);
+    zero2 += __shfl_xor(zero2, m, kWave);
     seen |= __shfl_xor(seen, m, kWave);
     seen2 |= __shfl_xor(seen2, m, kWave);
   }
   if ((threadIdx.x & 63) == 0) {
-    s_part[threadIdx.x >> 6] = local;
+    s_part[0][threadIdx.x >> 6] = local;
+    s_part[1][threadIdx.x >> 6] = zero;
+    s_part[2][threadIdx.x >> 6] = local2;
+    s_part[3][threadIdx.x >> 6] = zero2;
     s_mask[threadIdx.x >> 6] = seen;
     s_mask2[threadIdx.x >> 6] = seen2;
   }
   __syncthreads();
+  if (threadIdx.x < 4) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[threadIdx.x][w];
+    out[threadIdx.x * kHotCountSlots + blockIdx.x] = total;
+  }
   if (threadIdx.x == 0) {
-    int total = 0, m1 = 0, m2 = 0;
+    int m1 = 0, m2 = 0;
 #pragma unroll
     for (int w = 0; w < kWavesPerBlock; ++w) {
-      total += s_part[w];
       m1 |= s_mask[w];
       m2 |= s_mask2[w];
     }
-    out[blockIdx.x] = total;
     mask[blockIdx.x] = m1;
     mask[kHotCountSlots + blockIdx.x] = m2;
   }
@@ -552,7 +567,7 @@ publish_kernel(const float* __restrict__ A, const float* __restrict__ B, Shadow 
 size_t shadow_bytes() { return (size_t)kShadows * kHotWords * kMaxRounds * kWave * sizeof(float); }
 size_t shadow_counter_bytes() {
   return (size_t)2 * kShadows * kHotWords * kCounterStride * sizeof(unsigned) +
-         (size_t)3 * kHotCountSlots * sizeof(int);   // hot-word counts and the two id masks
+         (size_t)6 * kHotCountSlots * sizeof(int);   // four hot-word counts and the two id masks
 }
 size_t read_copy_bytes() { return (size_t)kXcds * kHotWords * kMaxRounds * kWave * sizeof(float); }
 
@@ -584,12 +599,14 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
                                        int waves_per_wg, Shadow* shadow) {
   const int mode = g_hot_update_mode.load();
   shadow->hot_total = 0;
+  shadow->hot_total_a = 0;
   if (A == nullptr || B == nullptr) shadow->pub_a = shadow->pub_b = nullptr;
   const bool forced = mode == kHotExact || mode == kHotCombining || mode == kHotOff;
   if (forced)
     shadow->combine = mode;
   else
     shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
+  shadow->combine_a = shadow->combine;
   if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
   if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
@@ -597,7 +614,10 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   // ids occur at all, for the read copies.
   hipLaunchKernelGGL(count_hot_kernel<Tables>, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids,
                      n, ids2, n2, tables, shadow->hot_seen, shadow->hot_mask);
-  if (!forced) shadow->hot_total = n;
+  if (!forced) {
+    shadow->hot_total = n;
+    shadow->hot_total_a = ids2 != nullptr ? n2 : 0;
+  }
   if (shadow->pub_a != nullptr)
     hipLaunchKernelGGL(publish_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, *shadow,
                        d);

@@ -82,6 +82,8 @@ class Word2Vec:
         self._ret = None
         self._call = 0
         self._wm = None
+        self._wm_last = None
+        self._prep = None
 
     # ---- Word2Vec.init ------------------------------------------------------------------
     def init(self, ncols=None, modelmats=None):
@@ -162,28 +164,66 @@ class Word2Vec:
 
     # ---- Word2Vec.wordMats (device branch) ----------------------------------------------
     def wordMatsDevice(self, mats):
-        """Same outputs as wordMats, as device tensors, built by the library on the GPU."""
+        """Same outputs as wordMats, as device tensors, built by the library on the GPU.
+
+        The upload and the preprocessing kernels run on a stream of their own, so that they are
+        not queued behind the update kernels of the previous minibatch, which the host has only
+        enqueued: the host prepares minibatch i+1 while the device still trains on minibatch i.
+        The outputs alternate between two sets of buffers; a set is written again only after the
+        update kernels that read it have finished (_release_index_arrays records that point), so
+        the tensors returned here stay valid until the call after next."""
         import torch
+        from .cumach import load_library
         o = self.opts
         wordsens = np.asarray(mats)
         n = wordsens.shape[1]
         cap = 2 * o.nskip * n
-        if self._wm is None or self._wm["n"] != n:
+        if self._wm is None or self._wm[0]["n"] != n:
             def ibuf(k):
                 return torch.empty(max(k, 1), dtype=torch.int32, device=self.device)
-            self._wm = dict(n=n, words=ibuf(n), lb=ibuf(n), ub=ibuf(n), ctx=ibuf(cap),
-                            negs=ibuf(o.nneg * (cap // o.nreuse + 1)), counts=ibuf(2))
-        b = self._wm
-        # the data source's 2 x n matrix, column-major: (word, sentence) pairs interleaved (no copy
-        # on the host if it already is, as matio.loadIMat returns it)
-        dmats = torch.from_numpy(np.ascontiguousarray(wordsens.T, dtype=np.int32)).to(self.device)
+            self._wm = [dict(n=n, words=ibuf(n), lb=ibuf(n), ub=ibuf(n), ctx=ibuf(cap),
+                             negs=ibuf(o.nneg * (cap // o.nreuse + 1)), counts=ibuf(2),
+                             free=None) for _ in range(2)]
+            self._prep = torch.cuda.Stream(device=self.device)
         self._call += 1
-        npairs, ngroups = _device_wordmats(n, dmats, o.iflip, o.vocabSize, o.nskip, o.nneg,
-                                           o.nreuse, float(np.float32(self.salpha)), o.wexpt,
-                                           o.seed, self._call, b["words"], b["lb"], b["ub"],
-                                           b["negs"], b["ctx"], b["counts"])
+        b = self._wm[self._call % 2]
+        self._wm_last = b
+        lib = load_library()
+        launch_stream = lib.w2v_get_stream()
+        with torch.cuda.stream(self._prep):
+            if b["free"] is not None:
+                self._prep.wait_event(b["free"])
+            # the data source's 2 x n matrix, column-major: (word, sentence) pairs interleaved (no
+            # copy on the host if it already is, as matio.loadIMat returns it)
+            dmats = torch.from_numpy(np.ascontiguousarray(wordsens.T, dtype=np.int32)).to(
+                self.device)
+            lib.w2v_set_stream(self._prep.cuda_stream)
+            try:
+                npairs, ngroups = _device_wordmats(n, dmats, o.iflip, o.vocabSize, o.nskip, o.nneg,
+                                                   o.nreuse, float(np.float32(self.salpha)),
+                                                   o.wexpt, o.seed, self._call, b["words"],
+                                                   b["lb"], b["ub"], b["negs"], b["ctx"],
+                                                   b["counts"])
+            finally:
+                lib.w2v_set_stream(launch_stream)
+        # w2v_wordmats has waited for its stream: the outputs are complete, whichever stream reads
+        # them next
         return (b["words"], b["lb"], b["ub"], b["negs"][:ngroups * o.nneg],
                 b["ctx"][:ngroups * o.nreuse])
+
+    def _release_index_arrays(self):
+        """Marks the point on the launch stream after which the buffers of the last
+        wordMatsDevice call may be overwritten (everything enqueued so far has read them)."""
+        import torch
+        b = getattr(self, "_wm_last", None)
+        if b is None:
+            return
+        if b["free"] is None:
+            b["free"] = torch.cuda.Event()
+        from .cumach import load_library
+        stream = load_library().w2v_get_stream()
+        b["free"].record(torch.cuda.ExternalStream(stream, device=self.device) if stream
+                         else torch.cuda.default_stream(self.device))
 
     def _index_arrays(self, mats):
         """(words, lb, ub, trandwords, contextwords) on the model's device."""
@@ -271,12 +311,13 @@ class Word2Vec:
             if goodwords.shape[0] > 0:
                 self.procNegativesSlice(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats,
                                         lrneg, o.vexp)
-            return
-        self.procPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0], lrpos,
-                           o.vexp)
-        if goodwords.shape[0] > 0:
-            self.procNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
-                               self.modelmats[0], lrneg, o.vexp)
+        else:
+            self.procPositives(o.nskip, words, lb, ub, self.modelmats[1], self.modelmats[0], lrpos,
+                               o.vexp)
+            if goodwords.shape[0] > 0:
+                self.procNegatives(o.nneg, o.nreuse, trandwords, goodwords, self.modelmats[1],
+                                   self.modelmats[0], lrneg, o.vexp)
+        self._release_index_arrays()
 
     def evalbatch(self, mats, ipass, pos):
         o = self.opts

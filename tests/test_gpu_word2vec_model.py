@@ -82,7 +82,7 @@ def test_device_wordmats_path_matches_oracle_step(oracle):
     m1 = m.modelmats[1].cpu().numpy().copy()
     mats = make_stream(6000, 4000, seed=21)
     m.dobatch(mats, 0, 6000)
-    b = m._wm
+    b = m._wm_last
     npairs, G = b["counts"].cpu().tolist()
     words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
     negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
@@ -122,7 +122,7 @@ def test_sliced_multipart_model_matches_oracle_step(oracle, dual):
     host = [x.cpu().numpy().copy() for x in m.modelmats]
     mats = make_stream(6000, 4000, seed=22)
     m.dobatch(mats, 0, 6000)
-    b = m._wm
+    b = m._wm_last
     npairs, G = b["counts"].cpu().tolist()
     words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
     negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
@@ -138,7 +138,7 @@ def test_sliced_multipart_model_matches_oracle_step(oracle, dual):
         assert np.array_equal(m.modelmats[1].cpu().numpy(), np.zeros_like(host[1]))
     held = make_stream(6000, 4000, seed=23)
     got = m.evalbatch(held, 0, 12000)
-    b = m._wm
+    b = m._wm_last
     npairs, G = b["counts"].cpu().tolist()
     words, lb, ub = (b[k].cpu().numpy() for k in ("words", "lb", "ub"))
     negs = b["negs"].cpu().numpy()[:G * o.nneg].copy()
