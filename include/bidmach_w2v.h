@@ -142,10 +142,12 @@ int w2v_get_max_workgroups(void);
  *      frequent word) from readers for a few microseconds; about 20 % faster than 0 on a raw
  *      Zipf stream;
  *   2  off: no shadow copies, every column is read and updated in place;
- *  -1  (default) decided per launch on the device: no shadow copies at all unless at least 1/16
- *      of the launch's word ids are among those 16 (they are not after frequent-word subsampling);
- *      otherwise combining for launches with at least 2048 wavefronts in flight, where that many
- *      updates are invisible to each other anyway, and exact for smaller ones. */
+ *  -1  (default) decided per launch and per table on the device: no shadow copies for a table
+ *      unless at least 1/16 of the word ids read from it are among those 16, or at least 1/48 are
+ *      id 0 (neither holds after frequent-word subsampling; the second holds for negatives drawn
+ *      with the reference's closed form, Word2Vec.scala:349-358); otherwise combining for launches
+ *      with at least 2048 wavefronts in flight, where that many updates are invisible to each
+ *      other anyway, and exact for smaller ones. */
 int w2v_set_hot_update_mode(int mode);
 int w2v_get_hot_update_mode(void);
 
