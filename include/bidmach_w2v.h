@@ -137,10 +137,11 @@ int w2v_get_max_workgroups(void);
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
  * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
  *   0  exact: their atomics are spread over shadow copies and every reader sums the copies;
- *   1  combining: readers read the table only and a copy is moved into the table on every 8th
- *      write to it, which hides fewer than 8 updates per copy (a couple of hundred of the most
- *      frequent word) from readers for a few microseconds; about 20 % faster than 0 on a raw
- *      Zipf stream;
+ *   1  combining: a copy is moved into the table on every 8th write to it, and readers read
+ *      neither the copies nor the table column but a per-XCD read copy of the column that every
+ *      such move refreshes; this hides fewer than 8 updates per copy (a couple of hundred of the
+ *      most frequent word) from readers for a few microseconds; about 20 % faster than 0 on a
+ *      raw Zipf stream;
  *   2  off: no shadow copies, every column is read and updated in place;
  *  -1  (default) decided per launch and per table on the device: no shadow copies for a table
  *      unless at least 1/16 of the word ids read from it are among those 16, or at least 1/48 are

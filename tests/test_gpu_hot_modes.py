@@ -76,6 +76,37 @@ def test_hot_columns_receive_every_update_exactly_once(gpu, hot_mode, d):
     assert np.abs(Bd.cpu().numpy() - B).max() < 5e-3 * np.abs(B).max()
 
 
+def test_default_mode_decides_per_table(gpu):
+    """No forced mode.  The words read from table B hold no hot id at all, a twentieth of those
+    read from table A are id 0 (what the reference's closed-form negative sampler does at a large
+    vocabulary): table A must get its shadow copies while table B goes without, and A's column 0
+    must still receive each of its 75,000 contributions exactly once (A starts at zero, so each is
+    -lr/2 times a sum of B columns to first order, whatever the interleaving)."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    assert load_library().w2v_get_hot_update_mode() == -1
+    rng = np.random.default_rng(21)
+    d, V, G, nwa, nwb = 64, 5000, 300000, 5, 5
+    A = np.zeros((V, d), np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    WA = rng.integers(16, V, G * nwa).astype(np.int32)
+    WA[rng.random(G * nwa) < 0.05] = 0
+    WB = rng.integers(16, V, G * nwb).astype(np.int32)
+    lr = 1e-7
+    Ad, Bd = parity.dev(torch, A), parity.dev(torch, B)
+    assert CUMACH.word2vecNeg(d, G, nwa, nwb, parity.dev(torch, WA), parity.dev(torch, WB), Ad, Bd,
+                              lr, 0.0) == 0
+    wa, wb = WA.reshape(G, nwa), WB.reshape(G, nwb)
+    sumB = B.astype(np.float64)[wb].sum(axis=1)                    # G x d
+    want = np.zeros((V, d))
+    np.add.at(want, wa.reshape(-1), np.repeat(-lr * 0.5 * sumB, nwa, axis=0))
+    got = Ad.cpu().numpy().astype(np.float64)
+    assert (wa == 0).sum() > 70000
+    scale0 = np.abs(want[0]).max()
+    assert np.abs(got[0] - want[0]).max() < 5e-3 * scale0
+    assert np.abs(got - want).max() < 5e-3 * np.abs(want).max()
+
+
 def test_mode_argument_is_normalised(gpu):
     from bidmach_amd.cumach import load_library
     lib = load_library()
