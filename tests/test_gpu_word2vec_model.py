@@ -94,6 +94,38 @@ def test_device_wordmats_path_matches_oracle_step(oracle):
     assert np.abs(m.modelmats[1].cpu().numpy() - m1).max() < 2e-3
 
 
+def test_back_to_back_minibatches_do_not_overwrite_index_arrays_in_use():
+    """dobatch only enqueues the update kernels, and the next call builds its index arrays on
+    another stream into the other buffer set: six different minibatches in a row, without waiting,
+    must train the same model as six calls that wait for the device after each one.  The second
+    table starts at zero and the step is tiny, so every update is, to first order, a sum that does
+    not depend on the order of the updates; index arrays overwritten while a kernel still reads them
+    would move whole contributions to other words."""
+    import torch
+
+    def run(wait):
+        o = Options(vocabSize=50000, dim=64, batchSize=200000, lrate=1e-5, vexp=0.0, texp=0.0,
+                    seed=9)
+        m = Word2Vec(o)
+        m.init()
+        stream = make_stream(200000 * 6, 50000, seed=31)
+        for k in range(6):
+            m.dobatch(stream[:, k * 200000:(k + 1) * 200000], 0, (k + 1) * 200000)
+            if wait:
+                m.synchronize()
+                torch.cuda.synchronize()
+        m.synchronize()
+        torch.cuda.synchronize()
+        return [x.cpu().numpy().astype(np.float64) for x in m.modelmats]
+
+    a0, a1 = run(False)
+    b0, b1 = run(True)
+    moved = np.abs(b1).max()                    # modelmats(1) starts at zero
+    assert moved > 1e-6
+    assert np.abs(a1 - b1).max() < 2e-2 * moved
+    assert np.abs(a0 - b0).max() < 2e-2 * moved
+
+
 def test_odd_sized_minibatch_is_skipped():
     import torch
     o = Options(vocabSize=500, dim=16, batchSize=1000, seed=1)
