@@ -350,6 +350,8 @@ hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, 
   if (most < 1) return hipSuccess;
   int every = 1;
   while (every < 8 && most / (2 * every) >= kRareMinSampledMax) every *= 2;
+  // a sample needs something to sample from (forced thresholds on small calls)
+  while (every > 1 && (na < nb ? na : nb) / (16 * every) < 4096) every /= 2;
   const int sampled_max = (int)(most / every);
   hipLaunchKernelGGL(clear_occurs_kernel, dim3(256), dim3(kBlock), 0, stream,
                      reinterpret_cast<int4*>(shadow->occurs), kOccurSlots / 4);
@@ -401,8 +403,11 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   hipError_t err = split_grid(reinterpret_cast<const void*>(kern), kNegThreads, 0, ngroups,
                               kMinGroupsPerWg, kMinGroupsPerWgWide, &g);
   if (err != hipSuccess) return err;
-  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa, A, B, d,
-                         g.nwg, kNegWaves, &shadow);
+  // word2vecNegFilt with fewer resident columns than hot ids: no read copies, which are filled
+  // from the columns of every hot id the launch holds, resident or not
+  const bool copies = idlimit >= kHotWords;
+  err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa,
+                         copies ? A : nullptr, copies ? B : nullptr, d, g.nwg, kNegWaves, &shadow);
   if (err != hipSuccess) return err;
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;
