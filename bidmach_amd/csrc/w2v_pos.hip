@@ -227,14 +227,19 @@ __host__ __device__ inline size_t tile_lds_bytes(int R, int T, int Sh) {
           2 * (size_t)(T + 2 * Sh)) * 4;
 }
 
+// Two buffers of 2*Sh columns for the B deltas a tile hands to the next one (see the kernel).
+__host__ __device__ inline size_t tile_carry_bytes(int R, int Sh) {
+  return (size_t)2 * (2 * Sh) * R * kWave * 4;
+}
+
 // `tables` is PlainTables (word2vecPos) or SlicedTables (word2vecPosSlice): it places a word's
 // column and says which pairs are trained and which columns are written.
 // Up to R = 7 two workgroups fit in a CU's LDS, which needs four waves per SIMD: the register
 // budget is held to that.
 template <int R, class Tables>
 __global__ void __launch_bounds__(kTileThreads, (R <= 7 ? 4 : 2))
-pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_per_wg_hot,
-                int64_t tiles_per_wg_wide,
+pos_tile_kernel(int d, int ncols, int T, int Sh, int carry, int64_t ntiles,
+                int64_t tiles_per_wg_hot, int64_t tiles_per_wg_wide,
                 const int* __restrict__ W, const int* __restrict__ LB,
                 const int* __restrict__ UB, Tables tables, float lrate, float vexp, int smode,
                 Shadow shadow_arg) {
@@ -249,10 +254,21 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
   float* const G = b_t + (size_t)(T + 2 * Sh) * dp;
   int* const wt = reinterpret_cast<int*>(G + (size_t)T * gw);
   int* const ft = wt + (T + 2 * Sh);
+  // Consecutive tiles of a workgroup overlap in 2*Sh staged positions (the last Sh centres of a
+  // tile and its trailing halo are the leading halo and the first Sh centres of the next).  With
+  // `carry` a tile does not scatter the B deltas of those positions but leaves them here, and the
+  // next tile adds its own share and scatters once: a position then costs one column of atomics
+  // instead of two.  Two buffers, because the waves that read the deltas handed in and the waves
+  // that write the deltas handed on run in the same phase.
+  float* const pend = reinterpret_cast<float*>(ft + (T + 2 * Sh));
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
-  const int64_t tiles_per_wg = launch_is_cold(shadow_arg, shadow) ? tiles_per_wg_wide
-                                                                   : tiles_per_wg_hot;
+  const bool cold = launch_is_cold(shadow_arg, shadow);
+  const int64_t tiles_per_wg = cold ? tiles_per_wg_wide : tiles_per_wg_hot;
+  // Measured: handing deltas on pays on launches without hot words (6 % on a subsampled stream),
+  // where many staged positions are empty and the atomics saved are a larger part of a tile's
+  // work; on a raw stream the longer second phase costs more than the atomics saved (7 %).
+  const bool carrying = carry != 0 && cold;
   const int64_t tile_begin = (int64_t)blockIdx.x * tiles_per_wg;
   const int64_t tile_end = min(tile_begin + tiles_per_wg, ntiles);
 
@@ -263,6 +279,12 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
     const int hhi = min(hi + Sh, ncols);        // staged positions [hlo, hhi)
     const int nh = hhi - hlo;
     const int nc = hi - lo;
+    // deltas handed in cover staged positions [0, 2*Sh); deltas handed on cover [c_out, nh)
+    const bool carry_in = carrying && tile > tile_begin;
+    const bool carry_out = carrying && tile + 1 < tile_end;
+    const int c_out = hi - Sh - hlo;
+    const float* const pend_in = pend + (size_t)(tile & 1) * (2 * Sh) * dp;
+    float* const pend_out = pend + (size_t)((tile + 1) & 1) * (2 * Sh) * dp;
 
     // ---- stage: word ids, B columns of every staged position, A columns of the centres.
     //      Two columns per wave are in flight at a time.
@@ -283,13 +305,20 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
           ft[c1] = r1.flags;
         }
       }
+      // what the previous tile computed for this position but has not written to the table yet
+      const bool in0 = carry_in && c0 < 2 * Sh && tables.written(r0.flags);
+      const bool in1 = carry_in && c1 < 2 * Sh && tables.written(r1.flags);
       if (r0.flags != 0) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) b_t[(size_t)c0 * dp + r * kWave + lane] = x0[r];
+        for (int r = 0; r < R; ++r)
+          b_t[(size_t)c0 * dp + r * kWave + lane] =
+              x0[r] + (in0 ? pend_in[(size_t)c0 * dp + r * kWave + lane] : 0.0f);
       }
       if (r1.flags != 0) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) b_t[(size_t)c1 * dp + r * kWave + lane] = x1[r];
+        for (int r = 0; r < R; ++r)
+          b_t[(size_t)c1 * dp + r * kWave + lane] =
+              x1[r] + (in1 ? pend_in[(size_t)c1 * dp + r * kWave + lane] : 0.0f);
       }
     }
     for (int c0 = wave; c0 < nc; c0 += 2 * kTileWaves) {
@@ -403,14 +432,16 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
         if (!tables.written(ft[c])) continue;
       }
       const int p = hlo + c;
+      const bool handed_in = carry_in && c < 2 * Sh;
+      const bool hand_on = carry_out && c >= c_out;
       // lane l looks at centre i = p - Sh + l; its g for this position sits at offset p - i
       const int i = p - Sh + lane;
       float gl = 0.0f;
       if (lane < gw && i >= lo && i < hi && i != p) gl = G[(i - lo) * gw + (p - i + Sh)];
       unsigned long long mask = __ballot(gl != 0.0f);
-      if (mask == 0ull) continue;
+      if (mask == 0ull && !handed_in && !hand_on) continue;
       const ColRef rp = tables.b(wp, d);
-      const unsigned tkb = lane == 0 ? hot_ticket(shadow, 0, slot, rp.hot) : 0u;
+      const unsigned tkb = (lane == 0 && !hand_on) ? hot_ticket(shadow, 0, slot, rp.hot) : 0u;
       float dbb[R];
       zero_col<R>(dbb);
       while (mask != 0ull) {
@@ -421,8 +452,19 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int64_t ntiles, int64_t tiles_p
 #pragma unroll
         for (int r = 0; r < R; ++r) dbb[r] = fmaf(g, acol[r * kWave], dbb[r]);
       }
-      scatter_axpy_ref<R>(rp, shadow, 0, slot, scale_of(wp, vexp, smode), dbb, lane, d,
-                          (unsigned)__builtin_amdgcn_readfirstlane((int)tkb));
+      const float bs = scale_of(wp, vexp, smode);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        dbb[r] *= bs;
+        if (handed_in) dbb[r] += pend_in[(size_t)c * dp + r * kWave + lane];
+      }
+      if (hand_on) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) pend_out[(size_t)(c - c_out) * dp + r * kWave + lane] = dbb[r];
+      } else {
+        scatter_add_ref<R>(rp, shadow, 0, slot, dbb, lane, d,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)tkb));
+      }
     }
     __syncthreads();
   }
@@ -770,7 +812,12 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   const int T = Sh > 0 ? pick_tile(R, Sh) : 0;
   *launched = T != 0;
   if (T == 0) return hipSuccess;
-  const size_t lds = tile_lds_bytes(R, T, Sh);
+  // Deltas are carried between tiles when the overlaps of consecutive tiles do not overlap each
+  // other and the extra LDS does not cost a workgroup per CU.
+  constexpr size_t kShareLds = 80 * 1024, kLimitLds = 160 * 1024;
+  const size_t base = tile_lds_bytes(R, T, Sh), with = base + tile_carry_bytes(R, Sh);
+  const int carry = (T >= 2 * Sh && with <= (base <= kShareLds ? kShareLds : kLimitLds)) ? 1 : 0;
+  const size_t lds = carry ? with : base;
   auto kern = pos_tile_kernel<R, Tables>;
   hipError_t err = hipSuccess;
   if (lds > 48 * 1024) {
@@ -793,7 +840,7 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   // only a launch that counts its hot words can turn out cold
   const int64_t nwg = shadow.hot_total > 0 ? g.nwg_wide : g.nwg;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kTileThreads), lds, stream, d, ncols, T, Sh,
-                     ntiles, g.per_wg, g.per_wg_wide, W, LB, UB, tables, lrate, vexp,
+                     carry, ntiles, g.per_wg, g.per_wg_wide, W, LB, UB, tables, lrate, vexp,
                      scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
