@@ -309,6 +309,8 @@ def main():
         out["roofline"]["traffic"] = None
     if args.hot_mode != -1:
         out["config"]["hot_update_mode"] = args.hot_mode
+    if args.rare_mode != -1:
+        out["config"]["rare_update_mode"] = args.rare_mode
     if args.wsample > 0.0:
         out["config"]["wsample"] = args.wsample
         out["roofline"]["traffic"] = None
