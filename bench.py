@@ -311,6 +311,8 @@ def main():
         out["config"]["hot_update_mode"] = args.hot_mode
     if args.rare_mode != -1:
         out["config"]["rare_update_mode"] = args.rare_mode
+    if args.tokens > 0:
+        out["roofline"]["traffic"] = None       # measured at the workload's own size only
     if args.wsample > 0.0:
         out["config"]["wsample"] = args.wsample
         out["roofline"]["traffic"] = None
