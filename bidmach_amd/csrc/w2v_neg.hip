@@ -330,13 +330,13 @@ int get_rare_update_mode() { return g_rare_update_mode.load(); }
 
 // Decides how many occurrences still make a word of this launch "rare" and counts the words.  A
 // launch of `units` work units keeps `waves` of them in flight, so a word with n occurrences has
-// about n * waves / units updates in flight together; words for which that is below 1/16 are
+// about n * waves / units updates in flight together; words for which that is below 1/8 are
 // updated without atomics.  Small launches get 0: everything stays atomic and nothing is counted.
 // The count is a scattered read-modify-write per id, which is what the device is slowest at, so for
 // thresholds that allow it only every 2nd, 4th or 8th run of ids is counted and the threshold
 // scaled down: the threshold is a soft one, and a word somewhat above it that slips through is as
 // harmless as one just below it.
-constexpr int kRareConcurrencyDen = 16;
+constexpr int kRareConcurrencyDen = 8;
 constexpr int kRareMaxCap = 64;
 constexpr int kRareMinSampledMax = 2;   // the scaled threshold is kept at or above this
 hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,

@@ -158,7 +158,7 @@ int w2v_get_hot_update_mode(void);
  * all threads (jni/src/BIDMach_CPUMACH.c:239-254).
  *   0  every update is a float atomic;
  *  -1, 1  (default) the call first counts, on the device, how often each word occurs in it; a word
- *      with so few occurrences that fewer than 1/16 of an update of it is in flight at any time, on
+ *      with so few occurrences that fewer than 1/8 of an update of it is in flight at any time, on
  *      average, is updated with a plain read-modify-write (bit-identical to the atomic update
  *      unless two updates of that column do overlap, in which case one of them is lost, as on the
  *      reference's CPU path).  Frequent words, and every word of a small call, stay atomic.  This
