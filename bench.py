@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # --pmc WRITE_SIZE on this same command (summaries under profiles/), scaled by what the same
 # counters read for a plain copy of known size in the same run (FETCH x2.0, WRITE x1.0).
 MEASURED_TRAFFIC_BYTES = {
-    "sgns_v1m_d300_w5_neg5_fp32": {"neg_kernel": 29.30e9, "pos_kernel": 4.74e9},
+    "sgns_v1m_d300_w5_neg5_fp32": {"neg_kernel": 29.35e9, "pos_kernel": 4.63e9},
 }
 
 WORKLOADS = {
