@@ -188,15 +188,16 @@ __device__ __forceinline__ void atomic_axpy_col(float* __restrict__ col, float a
 // between calls, so the same-line queue is spread over several lines.  A small kernel moves what
 // is left in the copies into the table at the end of the call.  Three modes (HotMode):
 //
-//   off: no shadow copies; every column is read and updated in place.  Chosen inside the kernel
-//       when the launch holds few hot words (fewer than 1/kHotShareDen of its ids, counted by a
-//       small kernel beforehand), as after frequent-word subsampling.
+//   off: no shadow copies; every column is read and updated in place.  Chosen inside the kernel,
+//       for each of the two tables, when the ids read from that table hold few hot words (counted
+//       by a small kernel beforehand, see ids_are_hot), as after frequent-word subsampling.
 //   exact (Shadow::combine == 0): while a pass runs, the value of hot column w is
 //       table[w] + sum of its copies, and a reader sums them all.  No update is delayed, but the
 //       readers of word 0 fetch 17 columns instead of one.  Words 0..7 are hot, with 16, 8, 8, 4,
 //       4, 4, 4, 2 copies (the Zipf shares).
-//   combining (Shadow::combine == 1): readers read the table column only.  What piles up in a
-//       copy is moved into the table by its writers: each copy has a write counter, and the
+//   combining (Shadow::combine == 1): readers read neither the copies nor the table column but a
+//       read copy of it (load_col_ref), or the table column where there are no read copies.  What
+//       piles up in a copy is moved into the table by its writers: each copy has a write counter, and the
 //       writer that brings it to a multiple of kFoldEvery swaps the copy to zero (an atomic
 //       exchange, so no concurrent add is lost or counted twice) and adds what it got to the
 //       table column.  A reader misses the updates parked in the copies, fewer than kFoldEvery
