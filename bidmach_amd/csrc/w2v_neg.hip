@@ -18,7 +18,10 @@
 // The update kernel is persistent: a fixed number of workgroups each walk a contiguous range of
 // groups, which bounds the number of groups in flight (and with it the staleness of the Hogwild
 // updates) by the launch size.  The atomics for the hottest columns go to their shadow copies
-// (w2v_device.h), so their same-line atomics spread over several lines.
+// (w2v_device.h), so their same-line atomics spread over several lines, and the columns of words
+// that are rare within the launch are updated with a device-scope read-modify-write instead of
+// atomics (prepare_rare_words below), which takes a third or more of the load off the float-atomic
+// units that bound the pass.
 //
 // The reference reads WA/WB without a validity test (:213-214,220-221); here a negative id
 // skips every pair it takes part in, so a bad id cannot become an out-of-bounds access.
