@@ -18,7 +18,8 @@ LIB_NAME = "libbidmachhip-linux-x86_64.so"
 LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
 PROBE_PATH = os.path.join(LIB_DIR, "probe_atomics")
 
-SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip", "w2v_api.hip"]
+SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
+           "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_api.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",

@@ -5,6 +5,7 @@
 #include <atomic>
 #include <cstring>
 
+#include "w2v_bf16.h"
 #include "w2v_internal.h"
 
 namespace {
@@ -353,6 +354,64 @@ int word2vecEvalPosAsync(int nrows, int ncols, int shift, int* W, int* LB, int* 
 int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A,
                          float* B, float* Retval) {
   return eval_neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, Retval, nullptr, false);
+}
+
+// ---- bfloat16 tables ------------------------------------------------------------------------
+
+int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, unsigned short* A,
+                    unsigned short* B, float lrate, float vexp, unsigned long long seed) {
+  (void)shift;
+  if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp,
+                                     seed),
+                true);
+}
+
+int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, unsigned short* A,
+                    unsigned short* B, float lrate, float vexp, unsigned long long seed) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb())
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
+                                     vexp, seed),
+                true);
+}
+
+int word2vecEvalPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB,
+                        unsigned short* A, unsigned short* B, double* Retval) {
+  (void)shift;
+  if (bad_common(nrows, ncols) || !Retval) return (int)hipErrorInvalidValue;
+  if (ncols == 0) return 0;
+  if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_eval_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B,
+                                          g_eval_floor.load(), Retval),
+                true);
+}
+
+int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
+                        unsigned short* A, unsigned short* B, double* Retval) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || !Retval)
+    return (int)hipErrorInvalidValue;
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_eval_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+                                          g_eval_floor.load(), Retval),
+                true);
+}
+
+int w2v_f32_to_bf16(size_t n, const float* src, unsigned short* dst) {
+  if (n == 0) return 0;
+  if (!src || !dst) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_f32_to_bf16(t_state.stream, n, src, dst), true);
+}
+
+int w2v_bf16_to_f32(size_t n, const unsigned short* src, float* dst) {
+  if (n == 0) return 0;
+  if (!src || !dst) return (int)hipErrorInvalidValue;
+  return finish(w2v::launch_bf16_to_f32(t_state.stream, n, src, dst), true);
 }
 
 void w2v_set_eval_floor(double floor_value) { g_eval_floor.store(floor_value); }

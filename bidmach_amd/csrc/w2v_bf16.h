@@ -1,0 +1,188 @@
+// Device-side building blocks of the reduced-precision storage variant: both tables are
+// bfloat16, every column is widened to fp32 when it is read, all arithmetic is the fp32 (double
+// inside exp / pow / log) arithmetic of the fp32 kernels, and a column is narrowed again with
+// stochastic rounding when it is written back.  There are no floating-point atomics on bf16
+// pairs that round stochastically, so the write-back is a compare-and-swap of the 4-byte word
+// (add_col16 below).
+//
+// Register layout: a column of d elements is held by the wave as RP = ceil(d / 128) element
+// pairs per lane: lane l holds elements 128 r + 2 l and 128 r + 2 l + 1.  With an even d and
+// 4-byte aligned tables every column starts on a 4-byte boundary, so a pair is one dword and each
+// memory instruction of the wave covers 256 contiguous bytes; otherwise the two halves are moved
+// separately.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "w2v_device.h"
+
+namespace w2v {
+
+constexpr int kMaxPairRounds = 10;  // d <= 1280, as for the fp32 tables
+
+// Dispatch on RP; a value without an instance of its own uses the next larger one (the extra
+// registers hold zeros and are never stored).
+#define W2V_PAIR_ROUNDS_SWITCH(RP_, CALL)                                                   \
+  switch (RP_) {                                                                            \
+    case 1: CALL(1); case 2: CALL(2); case 3: CALL(3); case 4: CALL(4); case 5: CALL(5);    \
+    case 6: CALL(6); case 7: case 8: CALL(8); case 9: case 10: CALL(10);                    \
+    default: return hipErrorInvalidValue;                                                   \
+  }
+
+__host__ __device__ __forceinline__ uint64_t sr_mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ULL;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+  return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ uint32_t sr_fmix32(uint32_t h) {
+  h ^= h >> 16;
+  h *= 0x85EBCA6BU;
+  h ^= h >> 13;
+  h *= 0xC2B2AE35U;
+  h ^= h >> 16;
+  return h;
+}
+
+// Key of one column write: `unit` is the token (positive pass) or group (negative pass) of the
+// call, `slot` the write inside it, `seed` the caller's seed of the call.
+__device__ __forceinline__ uint32_t sr_key(uint64_t seed, uint32_t unit, uint32_t slot) {
+  return (uint32_t)(sr_mix64(seed ^ sr_mix64(((uint64_t)unit << 32) | slot)) >> 32);
+}
+
+// fp32 -> bf16 with 16 random bits added below the kept mantissa: the magnitude rounds up with
+// probability (dropped bits) / 65536, so the expectation of the stored value is x.
+__device__ __forceinline__ uint32_t sr_narrow(float x, uint32_t key, uint32_t row) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  if ((u & 0x7F800000U) == 0x7F800000U)  // infinity or NaN: keep the class
+    return (u >> 16) | ((u & 0x007FFFFFU) ? 0x40U : 0U);
+  return (u + (sr_fmix32(key ^ (row * 0x9E3779B9U)) >> 16)) >> 16;
+}
+
+// Loads of the update kernels are device-scope (relaxed atomic loads): a plain
+// load may be served from the CU's own L1 or the XCD's own L2, which other CUs' and XCDs' stores
+// do not reach, so a wave that meets a frequent word again would read the column as it was the
+// first time and write back a sum that drops everything the rest of the device added since.
+// The forward kernels, which only read, use plain loads (DEVICE_SCOPE = false).
+template <bool DEVICE_SCOPE, typename T>
+__device__ __forceinline__ T load_elt(const T* p) {
+  if (DEVICE_SCOPE) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *p;
+}
+
+template <int RP, bool ALIGNED, bool DEVICE_SCOPE>
+__device__ __forceinline__ void load_col16(float (&x)[2 * RP], const uint16_t* col, int lane,
+                                           int d) {
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    const int e = r * 128 + 2 * lane;
+    if (ALIGNED) {
+      uint32_t v = 0;
+      if (e < d) v = load_elt<DEVICE_SCOPE>(reinterpret_cast<const uint32_t*>(col + e));
+      x[2 * r] = __builtin_bit_cast(float, v << 16);
+      x[2 * r + 1] = __builtin_bit_cast(float, v & 0xFFFF0000U);
+    } else {
+      const uint32_t lo = (e < d) ? load_elt<DEVICE_SCOPE>(col + e) : 0U;
+      const uint32_t hi = (e + 1 < d) ? load_elt<DEVICE_SCOPE>(col + e + 1) : 0U;
+      x[2 * r] = __builtin_bit_cast(float, lo << 16);
+      x[2 * r + 1] = __builtin_bit_cast(float, hi << 16);
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t cas_word(uint32_t* p, uint32_t expected, uint32_t desired) {
+  __hip_atomic_compare_exchange_strong(p, &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+  return expected;  // the value found: equal to the guess iff the exchange took place
+}
+
+// col[e] = narrow(widen(col[e]) + delta[e]) for the lane's elements, as a compare-and-swap on the
+// 4-byte word that holds them, so that no update of the column by another wave is lost: a store
+// of "what I read plus my delta" would wipe out whatever was added in between, and with
+// thousands of waves in flight the frequent words would lose most of their updates.  `seen` is
+// the column as this wave read it (the first guess; the exchange fails and is repeated with the
+// value found if the column has changed since).  The random bits depend on (key, row) only, so a
+// repeated attempt rounds the same way.
+template <int RP, bool ALIGNED>
+__device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 * RP],
+                                          const float (&delta)[2 * RP], int lane, int d,
+                                          uint32_t key) {
+  if (ALIGNED) {
+    uint32_t guess[RP], found[RP];
+    bool open[RP];
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      guess[r] = (__builtin_bit_cast(uint32_t, seen[2 * r]) >> 16) |
+                 (__builtin_bit_cast(uint32_t, seen[2 * r + 1]) & 0xFFFF0000U);
+      found[r] = guess[r];
+      open[r] = r * 128 + 2 * lane < d;
+    }
+    bool any = true;
+    while (any) {
+      // all of the lane's words are in flight together; only the ones that failed go again
+#pragma unroll
+      for (int r = 0; r < RP; ++r) {
+        if (open[r]) {
+          const int e = r * 128 + 2 * lane;
+          const float lo = __builtin_bit_cast(float, guess[r] << 16) + delta[2 * r];
+          const float hi = __builtin_bit_cast(float, guess[r] & 0xFFFF0000U) + delta[2 * r + 1];
+          const uint32_t want = sr_narrow(lo, key, (uint32_t)e) |
+                                (sr_narrow(hi, key, (uint32_t)(e + 1)) << 16);
+          found[r] = cas_word(reinterpret_cast<uint32_t*>(col + e), guess[r], want);
+        }
+      }
+      any = false;
+#pragma unroll
+      for (int r = 0; r < RP; ++r) {
+        if (open[r]) {
+          open[r] = found[r] != guess[r];
+          guess[r] = found[r];
+          any = any || open[r];
+        }
+      }
+    }
+  } else {
+    // columns on 2-byte boundaries: each element is exchanged inside the aligned word that
+    // holds it, the other half of the word being written back as found
+#pragma unroll
+    for (int r = 0; r < 2 * RP; ++r) {
+      const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
+      if (e < d) {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(col + e);
+        uint32_t* word = reinterpret_cast<uint32_t*>(addr & ~(uintptr_t)3);
+        const int shift = (addr & 2) ? 16 : 0;
+        uint32_t guess = load_elt<true>(word);
+        for (;;) {
+          const float x = __builtin_bit_cast(float, ((guess >> shift) & 0xFFFFU) << 16) + delta[r];
+          const uint32_t want = (guess & ~(0xFFFFU << shift)) |
+                                (sr_narrow(x, key, (uint32_t)e) << shift);
+          const uint32_t found = cas_word(word, guess, want);
+          if (found == guess) break;
+          guess = found;
+        }
+      }
+    }
+  }
+}
+
+// Launchers (enqueue only).  Tables are bf16, nrows x vocab, column-major.
+hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                           const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
+                           uint64_t seed);
+hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                           const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
+                           float vexp, uint64_t seed);
+// The forward twins add their sum into the device double Retval[0].
+hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W,
+                                const int* LB, const int* UB, const uint16_t* A,
+                                const uint16_t* B, double floorv, double* Retval);
+hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                const int* WA, const int* WB, const uint16_t* A,
+                                const uint16_t* B, double floorv, double* Retval);
+
+// Whole-table conversions: fp32 -> bf16 rounds to nearest, ties to even; bf16 -> fp32 is exact.
+hipError_t launch_f32_to_bf16(hipStream_t stream, size_t n, const float* src, uint16_t* dst);
+hipError_t launch_bf16_to_f32(hipStream_t stream, size_t n, const uint16_t* src, float* dst);
+
+}  // namespace w2v

@@ -1,0 +1,167 @@
+// Negative pass and its forward twin on bfloat16 tables (gfx950, wave64).
+//
+// One wavefront owns one group of nwa x nwb words.  It widens the group's nwb B columns into
+// registers, keeps an fp32 delta for each of them, and streams the nwa A columns through: each A
+// column is widened once, dotted with every B column (wave-level reduction), takes its own delta
+// from all of them and is written back at once, narrowed with stochastic rounding; the B columns
+// are written after the last A column.  All dots of a group therefore see the tables as they
+// were when the group started, which is what the reference's CPU loop computes for a group
+// without repeated words (jni/src/BIDMach_CPUMACH.c:210-254: A is written after every dot of the
+// group, a B column after its own dots).  A write-back adds the wave's delta to the column as
+// it is at that moment (compare-and-swap per 4-byte word), so concurrent updates of one column by
+// several waves are all kept.
+//
+// Every wave is persistent and walks a contiguous range of groups in order.
+#include "w2v_bf16.h"
+#include "w2v_internal.h"
+
+namespace w2v {
+
+namespace {
+
+constexpr int64_t kMinGroupsPerWave = 4;
+
+template <int RP, bool ALIGNED, int MAXB, bool EVAL>
+__global__ void __launch_bounds__(kBlock)
+neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __restrict__ WA,
+                const int* __restrict__ WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
+                int smode, uint64_t seed, double floorv, double* __restrict__ Retval) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
+  int64_t last = first + per_wave;
+  if (last > n) last = n;
+  double lsum = 0.0;
+  for (int64_t i = first; i < last; ++i) {
+    float b[MAXB][2 * RP], dbb[MAXB][2 * RP];
+    float bscale[MAXB];
+    int wb[MAXB];
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      wb[k] = 0;
+      bscale[k] = 0.0f;
+      if (k < nwb) {
+        wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
+        load_col16<RP, ALIGNED, !EVAL>(b[k], B + (int64_t)wb[k] * d, lane, d);
+        if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 2 * RP; ++r) b[k][r] = 0.0f;
+      }
+#pragma unroll
+      for (int r = 0; r < 2 * RP; ++r) dbb[k][r] = 0.0f;
+    }
+    for (int j = 0; j < nwa; ++j) {
+      const int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa + j]);
+      uint16_t* acol = A + (int64_t)wa * d;
+      float a[2 * RP], daa[2 * RP];
+      load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
+#pragma unroll
+      for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
+      const float ascale = EVAL ? 1.0f : scale_of(wa, vexp, smode);
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k) {
+        if (k < nwb) {
+          float part = 0.0f;
+#pragma unroll
+          for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[k][r], part);
+          const float sg = sat_sigmoid(wave_sum(part));
+          if (EVAL) {
+            lsum += log(fmax(1.0 - (double)sg, floorv));
+          } else {
+            const float g = -lrate * sg;
+            const float ga = ascale * g;
+            const float gb = bscale[k] * g;
+#pragma unroll
+            for (int r = 0; r < 2 * RP; ++r) {
+              dbb[k][r] = fmaf(gb, a[r], dbb[k][r]);
+              daa[r] = fmaf(ga, b[k][r], daa[r]);
+            }
+          }
+        }
+      }
+      if (!EVAL)
+        add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
+                               sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
+    }
+    if (!EVAL) {
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k) {
+        if (k < nwb)
+          add_col16<RP, ALIGNED>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
+                                 sr_key(seed, (uint32_t)i, (uint32_t)k));
+      }
+    }
+  }
+  if (EVAL) {
+    if (lane == 0 && lsum != 0.0) atomicAdd(Retval, lsum);
+  }
+}
+
+template <int RP, bool ALIGNED, int MAXB, bool EVAL>
+hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
+                  const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
+                  double floorv, double* Retval) {
+  auto kern = neg_bf16_kernel<RP, ALIGNED, MAXB, EVAL>;
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
+                                   kMinGroupsPerWave * kWavesPerBlock, &nwg);
+  if (err != hipSuccess) return err;
+  const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
+  nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, nwa, nwb,
+                     WA, WB, A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval);
+  return hipGetLastError();
+}
+
+template <bool ALIGNED, bool EVAL>
+hipError_t dispatch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
+                    const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
+                    uint64_t seed, double floorv, double* Retval) {
+  const int rp = (d + 127) / 128;
+  if (nwb <= 5) {
+#define W2V_CALL(RP_)                                                                         \
+  return launch<RP_, ALIGNED, 5, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
+                                       floorv, Retval)
+    W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+  }
+#define W2V_CALL(RP_)                                                                         \
+  return launch<RP_, ALIGNED, 8, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
+                                       floorv, Retval)
+  W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+}
+
+bool pair_aligned(int d, const void* A, const void* B) {
+  return (d & 1) == 0 && (reinterpret_cast<uintptr_t>(A) & 3) == 0 &&
+         (reinterpret_cast<uintptr_t>(B) & 3) == 0;
+}
+
+}  // namespace
+
+hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                           const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
+                           float vexp, uint64_t seed) {
+  if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
+  if (pair_aligned(nrows, A, B))
+    return dispatch<true, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
+                                 0.0, nullptr);
+  return dispatch<false, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
+                                0.0, nullptr);
+}
+
+hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                const int* WA, const int* WB, const uint16_t* A,
+                                const uint16_t* B, double floorv, double* Retval) {
+  if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
+  uint16_t* a = const_cast<uint16_t*>(A);  // the forward instance never stores
+  uint16_t* b = const_cast<uint16_t*>(B);
+  if (pair_aligned(nrows, A, B))
+    return dispatch<true, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0,
+                                floorv, Retval);
+  return dispatch<false, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0, floorv,
+                               Retval);
+}
+
+}  // namespace w2v

@@ -1,0 +1,184 @@
+// Positive pass and its forward twin on bfloat16 tables (gfx950, wave64).
+//
+// One wavefront owns one centre token.  It widens the centre's A column into registers, walks
+// the window, and for every valid context widens the B column, reduces the dot over the wave,
+// forms the fused sigmoid gradient, accumulates the centre's delta in fp32 registers and writes
+// the context column back at once, narrowed with stochastic rounding; the centre column is
+// written after the window.  That is the order of the reference's CPU loop
+// (jni/src/BIDMach_CPUMACH.c:29-67: B inside the window loop, A after it).  A write-back adds
+// the wave's delta to the column as it is at that moment (compare-and-swap per 4-byte word), so
+// concurrent updates of one column by several waves are all kept.
+//
+// Every wave is persistent and walks a contiguous range of tokens in order, as a thread of the
+// reference's CPU path does (:21-24): the overlapping windows of neighbouring tokens, which
+// rewrite the same context columns ten times over, are then handled by one wave one after the
+// other instead of by several waves at once, so those updates are not lost, and the re-read
+// columns are still in cache.
+#include "w2v_bf16.h"
+#include "w2v_internal.h"
+
+namespace w2v {
+
+namespace {
+
+constexpr int64_t kMinTokensPerWave = 16;
+
+template <int RP, bool ALIGNED, bool EVAL>
+__global__ void __launch_bounds__(kBlock)
+pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
+                const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A, uint16_t* B,
+                float lrate, float vexp, int smode, uint64_t seed, double floorv,
+                double* __restrict__ Retval) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
+  int64_t last = first + per_wave;
+  if (last > n) last = n;
+  double lsum = 0.0;
+  for (int64_t i = first; i < last; ++i) {
+    const int w = __builtin_amdgcn_readfirstlane(W[i]);
+    if (w < 0) continue;
+    const int lb = __builtin_amdgcn_readfirstlane(LB[i]);
+    const int ub = __builtin_amdgcn_readfirstlane(UB[i]);
+    uint16_t* acol = A + (int64_t)w * d;
+    float a[2 * RP], daa[2 * RP];
+    load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
+#pragma unroll
+    for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
+    const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
+    for (int j = lb; j <= ub; ++j) {
+      const int64_t p = i + j;
+      if (j == 0 || p < 0 || p >= n) continue;
+      const int wb = __builtin_amdgcn_readfirstlane(W[p]);
+      if (wb < 0) continue;
+      uint16_t* bcol = B + (int64_t)wb * d;
+      float b[2 * RP];
+      load_col16<RP, ALIGNED, !EVAL>(b, bcol, lane, d);
+      float part = 0.0f;
+#pragma unroll
+      for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[r], part);
+      const float sg = sat_sigmoid(wave_sum(part));
+      if (EVAL) {
+        lsum += log(fmax((double)sg, floorv));
+      } else {
+        const float g = lrate * (1.0f - sg);
+        const float ga = ascale * g;
+        const float gb = scale_of(wb, vexp, smode) * g;
+        float db[2 * RP];
+#pragma unroll
+        for (int r = 0; r < 2 * RP; ++r) {
+          daa[r] = fmaf(ga, b[r], daa[r]);
+          db[r] = gb * a[r];
+        }
+        add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
+      }
+    }
+    if (!EVAL) add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
+  }
+  if (EVAL) {
+    // lsum is wave-uniform; one double atomic per wave
+    if (lane == 0 && lsum != 0.0) atomicAdd(Retval, lsum);
+  }
+}
+
+template <int RP, bool ALIGNED, bool EVAL>
+hipError_t launch(hipStream_t stream, int d, int n, const int* W, const int* LB, const int* UB,
+                  uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed, double floorv,
+                  double* Retval) {
+  auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL>;
+  int64_t nwg = 0;
+  hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
+                                   kMinTokensPerWave * kWavesPerBlock, &nwg);
+  if (err != hipSuccess) return err;
+  const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
+  nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, W, LB, UB,
+                     A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval);
+  return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(kBlock)
+f32_to_bf16_kernel(size_t n, const float* __restrict__ src, uint16_t* __restrict__ dst) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, src[i]);
+    uint32_t h;
+    if ((u & 0x7F800000U) == 0x7F800000U)
+      h = (u >> 16) | ((u & 0x007FFFFFU) ? 0x40U : 0U);
+    else
+      h = (u + 0x7FFFU + ((u >> 16) & 1U)) >> 16;
+    dst[i] = (uint16_t)h;
+  }
+}
+
+__global__ void __launch_bounds__(kBlock)
+bf16_to_f32_kernel(size_t n, const uint16_t* __restrict__ src, float* __restrict__ dst) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+    dst[i] = __builtin_bit_cast(float, (uint32_t)src[i] << 16);
+}
+
+unsigned convert_grid(size_t n) {
+  size_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > 16384) blocks = 16384;
+  return (unsigned)blocks;
+}
+
+bool pair_aligned(int d, const void* A, const void* B) {
+  return (d & 1) == 0 && (reinterpret_cast<uintptr_t>(A) & 3) == 0 &&
+         (reinterpret_cast<uintptr_t>(B) & 3) == 0;
+}
+
+}  // namespace
+
+hipError_t launch_f32_to_bf16(hipStream_t stream, size_t n, const float* src, uint16_t* dst) {
+  hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(convert_grid(n)), dim3(kBlock), 0, stream, n, src,
+                     dst);
+  return hipGetLastError();
+}
+
+hipError_t launch_bf16_to_f32(hipStream_t stream, size_t n, const uint16_t* src, float* dst) {
+  hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(convert_grid(n)), dim3(kBlock), 0, stream, n, src,
+                     dst);
+  return hipGetLastError();
+}
+
+hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                           const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
+                           uint64_t seed) {
+  const int rp = (nrows + 127) / 128;
+  if (pair_aligned(nrows, A, B)) {
+#define W2V_CALL(RP_)                                                                          \
+  return launch<RP_, true, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
+                                  nullptr)
+    W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+  }
+#define W2V_CALL(RP_)                                                                           \
+  return launch<RP_, false, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
+                                   nullptr)
+  W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+}
+
+hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W,
+                                const int* LB, const int* UB, const uint16_t* A,
+                                const uint16_t* B, double floorv, double* Retval) {
+  const int rp = (nrows + 127) / 128;
+  uint16_t* a = const_cast<uint16_t*>(A);  // the forward instance never stores
+  uint16_t* b = const_cast<uint16_t*>(B);
+  if (pair_aligned(nrows, A, B)) {
+#define W2V_CALL(RP_)                                                                        \
+  return launch<RP_, true, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
+                                 Retval)
+    W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+  }
+#define W2V_CALL(RP_)                                                                         \
+  return launch<RP_, false, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
+                                  Retval)
+  W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
+#undef W2V_CALL
+}
+
+}  // namespace w2v

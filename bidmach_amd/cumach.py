@@ -52,6 +52,12 @@ SYMBOLS = {
     "word2vecNegAsync": (_I, _NEG),
     "word2vecEvalPosAsync": (_I, _EPOS),
     "word2vecEvalNegAsync": (_I, _ENEG),
+    "word2vecPosBf16": (_I, _POS + [ctypes.c_ulonglong]),
+    "word2vecNegBf16": (_I, _NEG + [ctypes.c_ulonglong]),
+    "word2vecEvalPosBf16": (_I, _EPOS),
+    "word2vecEvalNegBf16": (_I, _ENEG),
+    "w2v_f32_to_bf16": (_I, [_SZ, _P, _P]),
+    "w2v_bf16_to_f32": (_I, [_SZ, _P, _P]),
     "w2v_set_eval_floor": (None, [_D]),
     "w2v_get_eval_floor": (_D, []),
     "w2v_set_stream": (_I, [_P]),
@@ -242,6 +248,36 @@ class CUMACH:
     def word2vecEvalNegAsync(nrows, ncols, nwa, nwb, WA, WB, A, B, retVal):
         return load_library().word2vecEvalNegAsync(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB),
                                                    _ptr(A), _ptr(B), _ptr(retVal))
+
+    # -- bfloat16 tables (no Java counterpart): stochastic-rounded, atomic-free write-back -----
+
+    @staticmethod
+    def word2vecPosBf16(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, seed):
+        return load_library().word2vecPosBf16(nrows, ncols, shift, _ptr(W), _ptr(LB), _ptr(UB),
+                                              _ptr(A), _ptr(B), lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed):
+        return load_library().word2vecNegBf16(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB), _ptr(A),
+                                              _ptr(B), lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecEvalPosBf16(nrows, ncols, shift, W, LB, UB, A, B, retVal):
+        return load_library().word2vecEvalPosBf16(nrows, ncols, shift, _ptr(W), _ptr(LB),
+                                                  _ptr(UB), _ptr(A), _ptr(B), _ptr(retVal))
+
+    @staticmethod
+    def word2vecEvalNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, retVal):
+        return load_library().word2vecEvalNegBf16(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB),
+                                                  _ptr(A), _ptr(B), _ptr(retVal))
+
+
+def f32_to_bf16(n, src, dst):
+    check(load_library().w2v_f32_to_bf16(n, _ptr(src), _ptr(dst)), "w2v_f32_to_bf16")
+
+
+def bf16_to_f32(n, src, dst):
+    check(load_library().w2v_bf16_to_f32(n, _ptr(src), _ptr(dst)), "w2v_bf16_to_f32")
 
 
 def wordmats(n, mats, iflip, vocab, nskip, nneg, nreuse, wsample_lnv, wexpt, seed, call, words,

@@ -116,6 +116,36 @@ int word2vecEvalPosAsync(int nrows, int ncols, int shift, int *W, int *LB, int *
 int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
                          float *B, float *Retval);
 
+/* Reduced-precision storage: the four operators on bfloat16 tables (A and B are nrows x vocab,
+ * column-major, 2 bytes per element).  No counterpart in the reference, whose tables are fp32
+ * throughout; the argument lists are those of the four operators above with the element type
+ * changed, a seed added to the update calls and the forward sums added into a device double.
+ * A column is widened to fp32 when it is read; dots, sigmoid, scales and deltas are the fp32
+ * arithmetic of BIDMach_CPUMACH.c:10-78 / :186-264; a column is narrowed when it is written back,
+ * with stochastic rounding (the magnitude rounds up with probability dropped-bits / 65536, so the
+ * expectation of the stored value is the fp32 value) drawn from a counter-based generator keyed
+ * by `seed`, the token / group index, the write inside it and the row: pass a new seed for every
+ * call.  There is no floating-point atomic add on these tables: a write-back is a compare-and-swap
+ * of the 4-byte word that holds the elements, repeated with the value found when another update
+ * got there first, so concurrent updates of one column are all kept (a plain store of
+ * "value read + delta" loses most updates of the frequent words once thousands of work units are
+ * in flight).  With an odd nrows or a table on an odd 2-byte boundary the word that holds the
+ * first or last element of a table reaches 2 bytes outside it; those bytes are written back
+ * unchanged and must be addressable (they are inside any allocation the table is a view of).
+ * nwb <= w2v_max_nwb(). */
+int word2vecPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB, unsigned short *A,
+                    unsigned short *B, float lrate, float vexp, unsigned long long seed);
+int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, unsigned short *A,
+                    unsigned short *B, float lrate, float vexp, unsigned long long seed);
+int word2vecEvalPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB,
+                        unsigned short *A, unsigned short *B, double *Retval);
+int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB,
+                        unsigned short *A, unsigned short *B, double *Retval);
+/* Whole-table conversions between device buffers of n elements: fp32 -> bf16 rounds to nearest
+ * (ties to even), bf16 -> fp32 is exact.  Blocking. */
+int w2v_f32_to_bf16(size_t n, const float *src, unsigned short *dst);
+int w2v_bf16_to_f32(size_t n, const unsigned short *src, float *dst);
+
 /* Floor inside the Eval logarithms, process-wide.  Default 1e-40 (BIDMach_CPUMACH.c:409,467);
  * the reference's Scala and CUDA twins use 1e-20 (Word2Vec.scala:995,1123; DNN127.cu:310,916). */
 void w2v_set_eval_floor(double floor_value);

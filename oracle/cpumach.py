@@ -61,6 +61,20 @@ def _load():
                                                 ci, ci, ci, ci, ci]
     lib.oracle_word2vecEvalNegSlice.restype = cd
     lib.oracle_max_threads.restype = ci
+    hp = ctypes.POINTER(ctypes.c_uint16)
+    cu64, cu32 = ctypes.c_uint64, ctypes.c_uint32
+    lib.oracle_word2vecPosBf16.argtypes = [ci, ci, ci, ip, ip, ip, hp, hp, cf, cf, cu64]
+    lib.oracle_word2vecPosBf16.restype = None
+    lib.oracle_word2vecNegBf16.argtypes = [ci, ci, ci, ci, ip, ip, hp, hp, cf, cf, cu64]
+    lib.oracle_word2vecNegBf16.restype = None
+    lib.oracle_word2vecEvalPosBf16.argtypes = [ci, ci, ci, ip, ip, ip, hp, hp, cd]
+    lib.oracle_word2vecEvalPosBf16.restype = cd
+    lib.oracle_word2vecEvalNegBf16.argtypes = [ci, ci, ci, ci, ip, ip, hp, hp, cd]
+    lib.oracle_word2vecEvalNegBf16.restype = cd
+    lib.oracle_bf16_key.argtypes = [cu64, cu32, cu32]
+    lib.oracle_bf16_key.restype = cu32
+    lib.oracle_bf16_narrow.argtypes = [cf, cu32, cu32]
+    lib.oracle_bf16_narrow.restype = ctypes.c_uint16
     _lib = lib
     return lib
 
@@ -73,6 +87,29 @@ def _i(a):
 def _f(a):
     assert a.dtype == np.float32 and (a.flags.c_contiguous or a.flags.f_contiguous)
     return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def _h(a):
+    assert a.dtype == np.uint16 and (a.flags.c_contiguous or a.flags.f_contiguous)
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16))
+
+
+def bf16_widen(h):
+    """bfloat16 bit patterns (uint16) -> float32, exact."""
+    return (np.asarray(h, np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def bf16_truncate(x):
+    """float32 -> bfloat16 bit patterns by dropping the low 16 bits (round toward zero)."""
+    return (np.ascontiguousarray(x, np.float32).view(np.uint32) >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_key(seed, unit, slot):
+    return int(_load().oracle_bf16_key(seed, unit, slot))
+
+
+def bf16_narrow(x, key, row):
+    return int(_load().oracle_bf16_narrow(float(x), key, row))
 
 
 def _mm(mats):
@@ -119,6 +156,27 @@ class CPUMACH:
     def word2vecEvalNeg(nrows, ncols, nwa, nwb, WA, WB, A, B, nthreads, floor=C_FLOOR):
         return float(_load().oracle_word2vecEvalNeg(nrows, ncols, nwa, nwb, _i(WA), _i(WB),
                                                     _f(A), _f(B), floor, nthreads))
+
+    # ---- bfloat16 tables (no counterpart in the reference; oracle/w2v_oracle_bf16.c) ---------
+    @staticmethod
+    def word2vecPosBf16(nrows, ncols, skip, W, LB, UB, A, B, lrate, vexp, seed):
+        _load().oracle_word2vecPosBf16(nrows, ncols, skip, _i(W), _i(LB), _i(UB), _h(A), _h(B),
+                                       lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed):
+        _load().oracle_word2vecNegBf16(nrows, ncols, nwa, nwb, _i(WA), _i(WB), _h(A), _h(B),
+                                       lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecEvalPosBf16(nrows, ncols, skip, W, LB, UB, A, B, floor=C_FLOOR):
+        return float(_load().oracle_word2vecEvalPosBf16(nrows, ncols, skip, _i(W), _i(LB),
+                                                        _i(UB), _h(A), _h(B), floor))
+
+    @staticmethod
+    def word2vecEvalNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, floor=C_FLOOR):
+        return float(_load().oracle_word2vecEvalNegBf16(nrows, ncols, nwa, nwb, _i(WA), _i(WB),
+                                                        _h(A), _h(B), floor))
 
     # ---- sliced, multi-part models (CPUMACH.java:14,19; Scala-only forward twins) ----------
     @staticmethod

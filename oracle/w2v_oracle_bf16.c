@@ -1,0 +1,211 @@
+/*
+ * TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * CPU statement of the reduced-precision storage variant of the skip-gram negative-sampling
+ * functions: the same loop nests as oracle_word2vecPos / Neg / EvalPos / EvalNeg in
+ * w2v_oracle.c (which follow jni/src/BIDMach_CPUMACH.c:10-78, :186-264, :368-427, :429-483 of the
+ * reference), with both tables stored as bfloat16.  The reference has no such variant; what is
+ * kept from it is the arithmetic between a load and a store: every column is widened to fp32
+ * when it is read, dots, sigmoid, scales and deltas are the fp32 (double inside exp / pow / log)
+ * expressions of the reference, and a column is narrowed again only when it is written back.
+ *
+ * Narrowing is stochastic rounding with a counter-based generator, so that the HIP library and
+ * this file round every element with the same 16 random bits:
+ *   key  = mix64(seed ^ mix64((unit << 32) | slot))         unit = token / group index of the call
+ *   r16  = fmix32((uint32)(key >> 32) ^ (row * 0x9E3779B9)) >> 16
+ *   bf16 = (bits(x) + r16) >> 16                             (magnitude rounds up with
+ *                                                             probability low16(x) / 65536)
+ * slot names the write inside the unit: positive pass, context at offset j: (uint32)j, centre
+ * column: 0; negative pass, B column k: k, A column j: 0x10000 + j.
+ *
+ * Parity pins (tests/test_oracle_bf16.py): the narrowing is checked for its two neighbours and
+ * its mean (unbiased within sampling error) against numpy; on tables whose values are exactly
+ * representable and whose updates are exactly representable the result equals the fp32 oracle's;
+ * in general every element lies within one bf16 step of the fp32 oracle's result run on the
+ * widened tables; Eval equals the fp32 oracle's on the widened tables bit for bit.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+static inline float bf16_oracle_sigmoid(float cv) {
+  /* BIDMach_CPUMACH.c:48-55 */
+  if (cv > 16.0f) {
+    cv = 1.0f;
+  } else if (cv < -16.0f) {
+    cv = 0.0f;
+  } else {
+    cv = exp(cv);
+    cv = cv / (1.0f + cv);
+  }
+  return cv;
+}
+
+static inline float bf16_widen(uint16_t h) {
+  uint32_t u = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+static inline uint64_t bf16_mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ULL;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+  return z ^ (z >> 31);
+}
+
+static inline uint32_t bf16_fmix32(uint32_t h) {
+  h ^= h >> 16;
+  h *= 0x85EBCA6BU;
+  h ^= h >> 13;
+  h *= 0xC2B2AE35U;
+  h ^= h >> 16;
+  return h;
+}
+
+uint32_t oracle_bf16_key(uint64_t seed, uint32_t unit, uint32_t slot) {
+  return (uint32_t)(bf16_mix64(seed ^ bf16_mix64(((uint64_t)unit << 32) | slot)) >> 32);
+}
+
+uint16_t oracle_bf16_narrow(float x, uint32_t key, uint32_t row) {
+  uint32_t u;
+  memcpy(&u, &x, 4);
+  if ((u & 0x7F800000U) == 0x7F800000U) /* infinity or NaN: keep the class */
+    return (uint16_t)((u >> 16) | ((u & 0x007FFFFFU) ? 0x40U : 0U));
+  return (uint16_t)((u + (bf16_fmix32(key ^ (row * 0x9E3779B9U)) >> 16)) >> 16);
+}
+
+void oracle_word2vecPosBf16(int nrows, int ncols, int skip, const int *W, const int *LB,
+                            const int *UB, uint16_t *A, uint16_t *B, float lrate, float vexp,
+                            uint64_t seed) {
+  int i, j, c, itmp;
+  int64_t ia, ib;
+  float cv, ascale, bscale;
+  float *daa = (float *)malloc((size_t)nrows * sizeof(float));
+  (void)skip;
+  for (i = 0; i < ncols; i++) {
+    itmp = W[i];
+    if (itmp < 0) continue;
+    ia = (int64_t)nrows * itmp;
+    ascale = pow(1 + itmp, vexp);
+    for (c = 0; c < nrows; c++) daa[c] = 0;
+    for (j = LB[i]; j <= UB[i]; j++) {
+      if (j != 0 && i + j >= 0 && i + j < ncols) {
+        itmp = W[i + j];
+        if (itmp >= 0) {
+          uint32_t key = oracle_bf16_key(seed, (uint32_t)i, (uint32_t)j);
+          ib = (int64_t)nrows * itmp;
+          bscale = pow(1 + itmp, vexp);
+          cv = 0;
+          for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+          cv = bf16_oracle_sigmoid(cv);
+          cv = lrate * (1.0f - cv);
+          for (c = 0; c < nrows; c++) {
+            float a = bf16_widen(A[c + ia]), b = bf16_widen(B[c + ib]);
+            daa[c] += ascale * cv * b;
+            b += bscale * cv * a;
+            B[c + ib] = oracle_bf16_narrow(b, key, (uint32_t)c);
+          }
+        }
+      }
+    }
+    {
+      uint32_t key = oracle_bf16_key(seed, (uint32_t)i, 0U);
+      for (c = 0; c < nrows; c++)
+        A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c], key, (uint32_t)c);
+    }
+  }
+  free(daa);
+}
+
+void oracle_word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, const int *WA, const int *WB,
+                            uint16_t *A, uint16_t *B, float lrate, float vexp, uint64_t seed) {
+  int i, j, k, c, itmp;
+  int64_t ia, ib, ja;
+  float cv, ascale, bscale;
+  float *daa = (float *)malloc((size_t)(nwa > 0 ? nwa : 1) * nrows * sizeof(float));
+  float *dbb = (float *)malloc((size_t)nrows * sizeof(float));
+  for (i = 0; i < ncols; i++) {
+    for (c = 0; c < nwa * nrows; c++) daa[c] = 0;
+    for (k = 0; k < nwb; k++) {
+      uint32_t key = oracle_bf16_key(seed, (uint32_t)i, (uint32_t)k);
+      itmp = WB[k + (int64_t)i * nwb];
+      ib = (int64_t)nrows * itmp;
+      bscale = pow(1 + itmp, vexp);
+      for (c = 0; c < nrows; c++) dbb[c] = 0;
+      for (j = 0; j < nwa; j++) {
+        itmp = WA[j + (int64_t)i * nwa];
+        ia = (int64_t)nrows * itmp;
+        ascale = pow(1 + itmp, vexp);
+        cv = 0;
+        for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+        cv = bf16_oracle_sigmoid(cv);
+        cv = -lrate * cv;
+        ja = (int64_t)j * nrows;
+        for (c = 0; c < nrows; c++) {
+          dbb[c] += bscale * cv * bf16_widen(A[c + ia]);
+          daa[c + ja] += ascale * cv * bf16_widen(B[c + ib]);
+        }
+      }
+      for (c = 0; c < nrows; c++)
+        B[c + ib] = oracle_bf16_narrow(bf16_widen(B[c + ib]) + dbb[c], key, (uint32_t)c);
+    }
+    for (j = 0; j < nwa; j++) {
+      uint32_t key = oracle_bf16_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j);
+      ja = (int64_t)j * nrows;
+      ia = (int64_t)nrows * WA[j + (int64_t)i * nwa];
+      for (c = 0; c < nrows; c++)
+        A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c + ja], key, (uint32_t)c);
+    }
+  }
+  free(dbb);
+  free(daa);
+}
+
+double oracle_word2vecEvalPosBf16(int nrows, int ncols, int skip, const int *W, const int *LB,
+                                  const int *UB, const uint16_t *A, const uint16_t *B,
+                                  double floorv) {
+  int ii, j, c;
+  int64_t ia, ib;
+  float cv;
+  double dv = 0;
+  (void)skip;
+  for (ii = 0; ii < ncols; ii++) {
+    if (W[ii] < 0) continue;
+    ia = (int64_t)nrows * W[ii];
+    for (j = LB[ii]; j <= UB[ii]; j++) {
+      if (j != 0 && ii + j >= 0 && ii + j < ncols && W[ii + j] >= 0) {
+        ib = (int64_t)nrows * W[ii + j];
+        cv = 0;
+        for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+        cv = bf16_oracle_sigmoid(cv);
+        dv += log(fmax((double)cv, floorv));
+      }
+    }
+  }
+  return dv;
+}
+
+double oracle_word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, const int *WA,
+                                  const int *WB, const uint16_t *A, const uint16_t *B,
+                                  double floorv) {
+  int ii, j, k, c;
+  int64_t ia, ib;
+  float cv;
+  double dv = 0;
+  for (ii = 0; ii < ncols; ii++) {
+    for (k = 0; k < nwb; k++) {
+      ib = (int64_t)nrows * WB[k + (int64_t)ii * nwb];
+      for (j = 0; j < nwa; j++) {
+        ia = (int64_t)nrows * WA[j + (int64_t)ii * nwa];
+        cv = 0;
+        for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+        cv = bf16_oracle_sigmoid(cv);
+        dv += log(fmax(1.0 - (double)cv, floorv));
+      }
+    }
+  }
+  return dv;
+}
