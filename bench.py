@@ -37,6 +37,10 @@ WORKLOADS = {
                                          nneg=15, nreuse=5, zipf=1.0),
     "sgns_v10k_d100_w5_neg5_fp32": dict(vocab=10_000, dim=100, tokens=100_000, skip=5, nneg=5,
                                         nreuse=5, zipf=1.0),
+    # reduced-precision storage: bfloat16 tables, fp32 arithmetic, stochastic-rounded write-back
+    # (word2vecPosBf16 + word2vecNegBf16)
+    "sgns_v3m_d300_w5_neg5_bf16": dict(vocab=3_000_000, dim=300, tokens=1_000_000, skip=5, nneg=5,
+                                       nreuse=5, zipf=1.1, storage="bf16"),
     # forward-only scoring configuration (use with --mode eval)
     "sgns_v100k_d300_w5_neg5_fp32": dict(vocab=100_000, dim=300, tokens=1_000_000, skip=5, nneg=5,
                                          nreuse=5, zipf=1.0),
@@ -60,7 +64,7 @@ def make_minibatch(cfg, index, zcdf, ncdf, wsample=0.0):
 def algorithmic_bytes(cfg, mb):
     """Gather-scatter model: one read and one write of every column a work unit touches, plus the
     index arrays.  Pos: 2*C*(centres + pairs) + 12*N.  Neg: 2*C*G*(nwa+nwb) + 4*G*(nwa+nwb)."""
-    C = cfg["dim"] * 4
+    C = cfg["dim"] * (2 if cfg.get("storage") == "bf16" else 4)
     pos = 2 * C * (mb["centres"] + mb["pairs"]) + 12 * cfg["tokens"]
     k = cfg["nneg"] + cfg["nreuse"]
     neg = 2 * C * mb["G"] * k + 4 * mb["G"] * k
@@ -87,6 +91,27 @@ def cpu_baseline(cfg, mbs, lr_pos, lr_neg, vexp, threads):
                             lr_neg, vexp, threads)
     dt = time.perf_counter() - t0
     return len(mbs) * n / dt, dt
+
+
+def cpu_baseline_bf16(cfg, mb, lr_pos, lr_neg, vexp, tokens):
+    """Times the single-threaded bfloat16-storage oracle on the first `tokens` tokens of one
+    minibatch and the groups that go with them."""
+    from bidmach_amd import corpus
+    from oracle.cpumach import CPUMACH, bf16_truncate
+    d, n = cfg["dim"], cfg["tokens"]
+    B, A = corpus.init_tables(cfg["vocab"], d, seed=42)
+    A16, B16 = bf16_truncate(A), bf16_truncate(B)
+    del A, B
+    m = min(n, tokens)
+    g = int(mb["G"] * (m / float(n)))
+    W, LB, UB = mb["W"][:m].copy(), mb["LB"][:m].copy(), mb["UB"][:m].copy()
+    WA, WB = mb["WA"][:g * cfg["nneg"]].copy(), mb["WB"][:g * cfg["nreuse"]].copy()
+    CPUMACH.word2vecPosBf16(d, 2000, cfg["skip"], W, LB, UB, A16, B16, lr_pos, vexp, 1)  # warm-up
+    t0 = time.perf_counter()
+    CPUMACH.word2vecPosBf16(d, m, cfg["skip"], W, LB, UB, A16, B16, lr_pos, vexp, 2)
+    CPUMACH.word2vecNegBf16(d, g, cfg["nneg"], cfg["nreuse"], WA, WB, A16, B16, lr_neg, vexp, 3)
+    dt = time.perf_counter() - t0
+    return m / dt, dt, m
 
 
 def host_threads():
@@ -180,6 +205,17 @@ def main():
         return max(args.lrate * (1.0 - step / float(max(total, 1))), args.lrate * 1e-4)
 
     evaluating = args.mode == "eval"
+    bf16 = cfg.get("storage") == "bf16"
+    if bf16:
+        if evaluating or args.parts > 0:
+            sys.exit("bench.py: the bf16 workload runs in train mode on one unsliced model")
+        from bidmach_amd.cumach import f32_to_bf16
+        A16 = torch.empty(V * d, dtype=torch.int16, device="cuda")
+        B16 = torch.empty(V * d, dtype=torch.int16, device="cuda")
+        f32_to_bf16(V * d, A, A16)
+        f32_to_bf16(V * d, B, B16)
+        del A, B
+        A, B = A16, B16
     if evaluating:   # scoring needs non-trivial tables: N(0, 0.1) as the forward-only config says
         A.normal_(0.0, 0.1)
         B.normal_(0.0, 0.1)
@@ -205,6 +241,9 @@ def main():
         if evaluating:
             check(CUMACH.word2vecEvalPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B,
                                               ret[0:1]), "word2vecEvalPos")
+        elif bf16:   # blocking call; the timer brackets the kernel on the launch stream
+            check(CUMACH.word2vecPosBf16(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr,
+                                         args.vexp, 2 * s), "word2vecPosBf16")
         elif MM:
             check(CUMACH.word2vecPosSlice(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], MM, lr,
                                           args.vexp, 0, args.slices, maxcols, args.head, False, 1),
@@ -218,6 +257,10 @@ def main():
         if evaluating:
             check(CUMACH.word2vecEvalNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                               mb["WB"], A, B, ret[1:2]), "word2vecEvalNeg")
+        elif bf16:
+            check(CUMACH.word2vecNegBf16(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
+                                         mb["WB"], A, B, lr / cfg["nneg"], args.vexp, 2 * s + 1),
+                  "word2vecNegBf16")
         elif MM:
             check(CUMACH.word2vecNegSlice(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                           mb["WB"], MM, lr / cfg["nneg"], args.vexp, 0, args.slices,
@@ -260,7 +303,10 @@ def main():
     neg_gbps = avg_neg_b / (avg_neg_ms * 1e-3) / 1e9
     step_gbps = (avg_pos_b + avg_neg_b) / ((avg_pos_ms + avg_neg_ms) * 1e-3) / 1e9
 
-    assert bool(torch.isfinite(A).all()) and bool(torch.isfinite(B).all()), "tables diverged"
+    def finite(t):
+        return bool(torch.isfinite(t.view(torch.bfloat16) if bf16 else t).all())
+
+    assert finite(A) and finite(B), "tables diverged"
     if MM:
         assert all(bool(torch.isfinite(m).all()) for m in MM), "tables diverged"
 
@@ -279,7 +325,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32",   # arithmetic type; the bf16 workload stores bf16 and computes in fp32
         "data": "synthetic",
         "config": {"workload": args.workload, "vocab": V, "dim": d, "tokens_per_minibatch": n,
                    "window": cfg["skip"], "nneg": cfg["nneg"], "nreuse": cfg["nreuse"],
@@ -307,6 +353,9 @@ def main():
     if evaluating:
         out["config"]["mode"] = "eval"
         out["roofline"]["traffic"] = None
+    if bf16:
+        out["config"]["storage"] = "bf16"
+        out["config"]["operators"] = "word2vecPosBf16+word2vecNegBf16"
     if args.hot_mode != -1:
         out["config"]["hot_update_mode"] = args.hot_mode
     if args.rare_mode != -1:
@@ -322,7 +371,7 @@ def main():
         out["config"]["head_words"] = args.head
         out["config"]["operators"] = "word2vecPosSlice+word2vecNegSlice"
         out["roofline"]["traffic"] = None
-    if not evaluating and not MM and not args.no_pcie:
+    if not evaluating and not MM and not bf16 and not args.no_pcie:
         # The same step with the five index arrays uploaded from pinned host memory first (what a
         # caller that builds them on the host pays); serialised with the kernels, not overlapped.
         # Reported beside the headline value, never as it.
@@ -363,7 +412,15 @@ def main():
     out["hbm_copy"] = {"achieved": copy_gbps, "unit": "GB/s read+write",
                        "step_algorithmic_over_copy": step_gbps / copy_gbps}
 
-    if not args.no_cpu_baseline and not evaluating:
+    if not args.no_cpu_baseline and bf16:
+        cpu_wps, cpu_dt, m = cpu_baseline_bf16(cfg, host_mbs[0], args.lrate,
+                                               args.lrate / cfg["nneg"], args.vexp, 300_000)
+        out["cpu_baseline"] = {"value": cpu_wps, "unit": "words/s", "cores": 1, "kind": "port",
+                               "sample": "the first %d tokens of one minibatch and their groups, "
+                                         "pos+neg, single-threaded bf16 oracle, %.1f s wall"
+                                         % (m, cpu_dt),
+                               "gpu_over_cpu": words_per_s / cpu_wps}
+    elif not args.no_cpu_baseline and not evaluating:
         threads = host_threads()
         sample = host_mbs[:3]
         cpu_wps, cpu_dt = cpu_baseline(cfg, sample, args.lrate, args.lrate / cfg["nneg"],

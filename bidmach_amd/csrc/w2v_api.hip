@@ -18,11 +18,54 @@ struct ThreadState {
   double* partials[kMaxDevices] = {};
   int64_t capacity[kMaxDevices] = {};
   float* shadow[kMaxDevices] = {};  // two shadow buffers (A then B), zero between calls
+  float* side16[kMaxDevices] = {};  // fp32 side buffers of the bf16 tables' frequent words
+  size_t side16_floats[kMaxDevices] = {};
 };
 
 thread_local ThreadState t_state;
 
 std::atomic<double> g_eval_floor{1.0e-40};
+std::atomic<int> g_bf16_hot_words{1024};
+constexpr int kMaxBf16HotWords = 4096;
+
+// Per-thread, per-device fp32 side buffers for the frequent words of bf16 tables (A's then B's),
+// zeroed when allocated; the update launchers leave them zeroed.  They only grow.
+hipError_t side_buffers(int nrows, w2v::HotCols* out) {
+  const int n = g_bf16_hot_words.load();
+  out->n = n;
+  out->sa = out->sb = nullptr;
+  if (n == 0) return hipSuccess;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  ThreadState& ts = t_state;
+  const size_t need = (size_t)2 * n * nrows;
+  if (ts.side16_floats[dev] < need) {
+    if (ts.side16[dev] != nullptr) {
+      err = hipStreamSynchronize(ts.stream);
+      if (err != hipSuccess) return err;
+      err = hipFree(ts.side16[dev]);
+      ts.side16[dev] = nullptr;
+      ts.side16_floats[dev] = 0;
+      if (err != hipSuccess) return err;
+    }
+    float* p = nullptr;
+    err = hipMalloc(reinterpret_cast<void**>(&p), need * sizeof(float));
+    if (err != hipSuccess) return err;
+    err = hipMemsetAsync(p, 0, need * sizeof(float), ts.stream);
+    if (err == hipSuccess) err = hipStreamSynchronize(ts.stream);
+    if (err != hipSuccess) {
+      (void)hipFree(p);
+      return err;
+    }
+    ts.side16[dev] = p;
+    ts.side16_floats[dev] = need;
+  }
+  out->sa = ts.side16[dev];
+  out->sb = ts.side16[dev] + (size_t)n * nrows;
+  return hipSuccess;
+}
 
 // Per-thread, per-device buffer of per-block partial sums for the Eval kernels.  It only grows.
 hipError_t eval_scratch(int64_t need, double** out) {
@@ -364,8 +407,11 @@ int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, u
   if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  w2v::HotCols hot{};
+  hipError_t err = side_buffers(nrows, &hot);
+  if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp,
-                                     seed),
+                                     seed, hot),
                 true);
 }
 
@@ -375,8 +421,11 @@ int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, un
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  w2v::HotCols hot{};
+  hipError_t err = side_buffers(nrows, &hot);
+  if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
-                                     vexp, seed),
+                                     vexp, seed, hot),
                 true);
 }
 
@@ -401,6 +450,13 @@ int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB
                                           g_eval_floor.load(), Retval),
                 true);
 }
+
+int w2v_set_bf16_hot_words(int n) {
+  if (n < 0 || n > kMaxBf16HotWords) return (int)hipErrorInvalidValue;
+  g_bf16_hot_words.store(n);
+  return 0;
+}
+int w2v_get_bf16_hot_words(void) { return g_bf16_hot_words.load(); }
 
 int w2v_f32_to_bf16(size_t n, const float* src, unsigned short* dst) {
   if (n == 0) return 0;

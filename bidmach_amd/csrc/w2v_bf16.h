@@ -166,13 +166,57 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
   }
 }
 
+// Frequent words.  Word ids are frequency ranks, so the first few hundred ids take most of the
+// updates of a call, and a compare-and-swap on a column that thousands of waves update at once
+// fails nearly every time.  The columns of the words below `n` therefore have an fp32 side
+// buffer each (sa for table A, sb for table B; n x d floats, zero between calls): while a call
+// runs, the value of such a column is widen(table) + side buffer, readers add the two in fp32,
+// and writers add their delta to the side buffer with float atomics, which need no retry.  A small
+// kernel at the end of the call narrows table + side buffer back into the table (one stochastic
+// rounding per element and call instead of one per update) and clears the side buffer.
+struct HotCols {
+  float* sa;
+  float* sb;
+  int n;
+};
+
+template <int RP>
+__device__ __forceinline__ void add_side_col(float (&x)[2 * RP], const float* side, int lane,
+                                             int d) {
+#pragma unroll
+  for (int r = 0; r < 2 * RP; ++r) {
+    const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
+    if (e < d) x[r] += __hip_atomic_load(side + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int RP>
+__device__ __forceinline__ void atomic_add_side_col(float* side, const float (&delta)[2 * RP],
+                                                    int lane, int d) {
+#pragma unroll
+  for (int r = 0; r < 2 * RP; ++r) {
+    const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
+    if (e < d) atomicAdd(side + e, delta[r]);
+  }
+}
+
+// Slot of the end-of-call narrowing of a frequent word's column in the random-bit key (the unit
+// is 0xFFFFFFFF, which no token or group index reaches).
+__host__ __device__ __forceinline__ uint32_t fold_slot(int table_b, int word) {
+  return ((uint32_t)table_b << 31) | (uint32_t)word;
+}
+
 // Launchers (enqueue only).  Tables are bf16, nrows x vocab, column-major.
+// `hot` holds zeroed side buffers of hot.n x nrows floats each (hot.n may be 0); the update
+// launchers leave them zeroed (they enqueue the narrowing kernel after the update kernel).
 hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
                            const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                           uint64_t seed);
+                           uint64_t seed, HotCols hot);
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
-                           float vexp, uint64_t seed);
+                           float vexp, uint64_t seed, HotCols hot);
+hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
+                            HotCols hot);
 // The forward twins add their sum into the device double Retval[0].
 hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W,
                                 const int* LB, const int* UB, const uint16_t* A,

@@ -25,7 +25,8 @@ template <int RP, bool ALIGNED, int MAXB, bool EVAL>
 __global__ void __launch_bounds__(kBlock)
 neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __restrict__ WA,
                 const int* __restrict__ WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                int smode, uint64_t seed, double floorv, double* __restrict__ Retval) {
+                int smode, uint64_t seed, double floorv, double* __restrict__ Retval,
+                HotCols hot) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
@@ -43,6 +44,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       if (k < nwb) {
         wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
         load_col16<RP, ALIGNED, !EVAL>(b[k], B + (int64_t)wb[k] * d, lane, d);
+        if (!EVAL && wb[k] < hot.n) add_side_col<RP>(b[k], hot.sb + (int64_t)wb[k] * d, lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
       } else {
 #pragma unroll
@@ -56,6 +58,8 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       uint16_t* acol = A + (int64_t)wa * d;
       float a[2 * RP], daa[2 * RP];
       load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
+      const bool ahot = !EVAL && wa < hot.n;
+      if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)wa * d, lane, d);
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
       const float ascale = EVAL ? 1.0f : scale_of(wa, vexp, smode);
@@ -80,16 +84,24 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
           }
         }
       }
-      if (!EVAL)
-        add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
-                               sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
+      if (!EVAL) {
+        if (ahot)
+          atomic_add_side_col<RP>(hot.sa + (int64_t)wa * d, daa, lane, d);
+        else
+          add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
+                                 sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
+      }
     }
     if (!EVAL) {
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
-        if (k < nwb)
-          add_col16<RP, ALIGNED>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
-                                 sr_key(seed, (uint32_t)i, (uint32_t)k));
+        if (k < nwb) {
+          if (wb[k] < hot.n)
+            atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
+          else
+            add_col16<RP, ALIGNED>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
+                                   sr_key(seed, (uint32_t)i, (uint32_t)k));
+        }
       }
     }
   }
@@ -101,7 +113,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
 template <int RP, bool ALIGNED, int MAXB, bool EVAL>
 hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
                   const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
-                  double floorv, double* Retval) {
+                  double floorv, double* Retval, HotCols hot) {
   auto kern = neg_bf16_kernel<RP, ALIGNED, MAXB, EVAL>;
   int64_t nwg = 0;
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
@@ -110,25 +122,27 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
   const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
   nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, nwa, nwb,
-                     WA, WB, A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval);
-  return hipGetLastError();
+                     WA, WB, A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval, hot);
+  hipError_t lerr = hipGetLastError();
+  if (lerr != hipSuccess || EVAL || hot.n == 0) return lerr;
+  return launch_fold_bf16(stream, d, A, B, seed, hot);
 }
 
 template <bool ALIGNED, bool EVAL>
 hipError_t dispatch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
                     const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                    uint64_t seed, double floorv, double* Retval) {
+                    uint64_t seed, double floorv, double* Retval, HotCols hot) {
   const int rp = (d + 127) / 128;
   if (nwb <= 5) {
 #define W2V_CALL(RP_)                                                                         \
   return launch<RP_, ALIGNED, 5, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
-                                       floorv, Retval)
+                                       floorv, Retval, hot)
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
 #define W2V_CALL(RP_)                                                                         \
   return launch<RP_, ALIGNED, 8, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
-                                       floorv, Retval)
+                                       floorv, Retval, hot)
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }
@@ -142,13 +156,13 @@ bool pair_aligned(int d, const void* A, const void* B) {
 
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
-                           float vexp, uint64_t seed) {
+                           float vexp, uint64_t seed, HotCols hot) {
   if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
   if (pair_aligned(nrows, A, B))
     return dispatch<true, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
-                                 0.0, nullptr);
+                                 0.0, nullptr, hot);
   return dispatch<false, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
-                                0.0, nullptr);
+                                0.0, nullptr, hot);
 }
 
 hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
@@ -159,9 +173,9 @@ hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nw
   uint16_t* b = const_cast<uint16_t*>(B);
   if (pair_aligned(nrows, A, B))
     return dispatch<true, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0,
-                                floorv, Retval);
+                                floorv, Retval, HotCols{});
   return dispatch<false, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0, floorv,
-                               Retval);
+                               Retval, HotCols{});
 }
 
 }  // namespace w2v

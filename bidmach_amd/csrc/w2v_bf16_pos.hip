@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(kBlock)
 pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
                 const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A, uint16_t* B,
                 float lrate, float vexp, int smode, uint64_t seed, double floorv,
-                double* __restrict__ Retval) {
+                double* __restrict__ Retval, HotCols hot) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
@@ -43,6 +43,8 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     uint16_t* acol = A + (int64_t)w * d;
     float a[2 * RP], daa[2 * RP];
     load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
+    const bool ahot = !EVAL && w < hot.n;
+    if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)w * d, lane, d);
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
@@ -54,6 +56,8 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       uint16_t* bcol = B + (int64_t)wb * d;
       float b[2 * RP];
       load_col16<RP, ALIGNED, !EVAL>(b, bcol, lane, d);
+      const bool bhot = !EVAL && wb < hot.n;
+      if (bhot) add_side_col<RP>(b, hot.sb + (int64_t)wb * d, lane, d);
       float part = 0.0f;
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[r], part);
@@ -70,10 +74,18 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
           daa[r] = fmaf(ga, b[r], daa[r]);
           db[r] = gb * a[r];
         }
-        add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
+        if (bhot)
+          atomic_add_side_col<RP>(hot.sb + (int64_t)wb * d, db, lane, d);
+        else
+          add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
     }
-    if (!EVAL) add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
+    if (!EVAL) {
+      if (ahot)
+        atomic_add_side_col<RP>(hot.sa + (int64_t)w * d, daa, lane, d);
+      else
+        add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
+    }
   }
   if (EVAL) {
     // lsum is wave-uniform; one double atomic per wave
@@ -84,7 +96,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
 template <int RP, bool ALIGNED, bool EVAL>
 hipError_t launch(hipStream_t stream, int d, int n, const int* W, const int* LB, const int* UB,
                   uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed, double floorv,
-                  double* Retval) {
+                  double* Retval, HotCols hot) {
   auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL>;
   int64_t nwg = 0;
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
@@ -93,8 +105,30 @@ hipError_t launch(hipStream_t stream, int d, int n, const int* W, const int* LB,
   const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
   nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, W, LB, UB,
-                     A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval);
-  return hipGetLastError();
+                     A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval, hot);
+  hipError_t lerr = hipGetLastError();
+  if (lerr != hipSuccess || EVAL || hot.n == 0) return lerr;
+  return launch_fold_bf16(stream, d, A, B, seed, hot);
+}
+
+// One workgroup per frequent word and table: table column = narrow(widen(column) + side buffer),
+// side buffer = 0.  Elements whose side buffer is zero are left alone, so a word the call did not
+// update keeps its bits (and a word id beyond the vocabulary is never touched).
+__global__ void __launch_bounds__(kBlock)
+fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot) {
+  const int w = blockIdx.x >> 1;
+  const int table_b = blockIdx.x & 1;
+  uint16_t* col = (table_b ? B : A) + (int64_t)w * d;
+  float* side = (table_b ? hot.sb : hot.sa) + (int64_t)w * d;
+  const uint32_t key = sr_key(seed, 0xFFFFFFFFU, fold_slot(table_b, w));
+  for (int e = threadIdx.x; e < d; e += kBlock) {
+    const float v = side[e];
+    if (v != 0.0f) {
+      const float x = __builtin_bit_cast(float, (uint32_t)col[e] << 16) + v;
+      col[e] = (uint16_t)sr_narrow(x, key, (uint32_t)e);
+      side[e] = 0.0f;
+    }
+  }
 }
 
 __global__ void __launch_bounds__(kBlock)
@@ -143,20 +177,28 @@ hipError_t launch_bf16_to_f32(hipStream_t stream, size_t n, const uint16_t* src,
   return hipGetLastError();
 }
 
+hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
+                            HotCols hot) {
+  if (hot.n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(fold_bf16_kernel, dim3(2u * (unsigned)hot.n), dim3(kBlock), 0, stream, nrows,
+                     A, B, seed, hot);
+  return hipGetLastError();
+}
+
 hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
                            const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                           uint64_t seed) {
+                           uint64_t seed, HotCols hot) {
   const int rp = (nrows + 127) / 128;
   if (pair_aligned(nrows, A, B)) {
 #define W2V_CALL(RP_)                                                                          \
   return launch<RP_, true, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
-                                  nullptr)
+                                  nullptr, hot)
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
 #define W2V_CALL(RP_)                                                                           \
   return launch<RP_, false, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
-                                   nullptr)
+                                   nullptr, hot)
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }
@@ -170,13 +212,13 @@ hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const 
   if (pair_aligned(nrows, A, B)) {
 #define W2V_CALL(RP_)                                                                        \
   return launch<RP_, true, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
-                                 Retval)
+                                 Retval, HotCols{})
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
 #define W2V_CALL(RP_)                                                                         \
   return launch<RP_, false, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
-                                  Retval)
+                                  Retval, HotCols{})
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }

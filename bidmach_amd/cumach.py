@@ -56,6 +56,8 @@ SYMBOLS = {
     "word2vecNegBf16": (_I, _NEG + [ctypes.c_ulonglong]),
     "word2vecEvalPosBf16": (_I, _EPOS),
     "word2vecEvalNegBf16": (_I, _ENEG),
+    "w2v_set_bf16_hot_words": (_I, [_I]),
+    "w2v_get_bf16_hot_words": (_I, []),
     "w2v_f32_to_bf16": (_I, [_SZ, _P, _P]),
     "w2v_bf16_to_f32": (_I, [_SZ, _P, _P]),
     "w2v_set_eval_floor": (None, [_D]),

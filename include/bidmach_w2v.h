@@ -141,6 +141,16 @@ int word2vecEvalPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *U
                         unsigned short *A, unsigned short *B, double *Retval);
 int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB,
                         unsigned short *A, unsigned short *B, double *Retval);
+/* Number of frequent words (ids 0 .. n-1; ids are frequency ranks) whose bf16 columns are updated
+ * through an fp32 side buffer during a call: readers add table and side buffer in fp32, writers
+ * add their delta to the side buffer with float atomics, and the end of the call narrows the sum
+ * back into the table with one stochastic rounding per element (slot: unit 0xFFFFFFFF of the
+ * generator).  A compare-and-swap on a column that thousands of work units update at once fails
+ * nearly every time; float atomics need no retry.  Default 1024, at most 4096, 0 = every column
+ * by compare-and-swap.  Process-wide; the side buffers belong to the calling thread. */
+int w2v_set_bf16_hot_words(int n);
+int w2v_get_bf16_hot_words(void);
+
 /* Whole-table conversions between device buffers of n elements: fp32 -> bf16 rounds to nearest
  * (ties to even), bf16 -> fp32 is exact.  Blocking. */
 int w2v_f32_to_bf16(size_t n, const float *src, unsigned short *dst);

@@ -63,9 +63,9 @@ def _load():
     lib.oracle_max_threads.restype = ci
     hp = ctypes.POINTER(ctypes.c_uint16)
     cu64, cu32 = ctypes.c_uint64, ctypes.c_uint32
-    lib.oracle_word2vecPosBf16.argtypes = [ci, ci, ci, ip, ip, ip, hp, hp, cf, cf, cu64]
+    lib.oracle_word2vecPosBf16.argtypes = [ci, ci, ci, ip, ip, ip, hp, hp, cf, cf, cu64, ci]
     lib.oracle_word2vecPosBf16.restype = None
-    lib.oracle_word2vecNegBf16.argtypes = [ci, ci, ci, ci, ip, ip, hp, hp, cf, cf, cu64]
+    lib.oracle_word2vecNegBf16.argtypes = [ci, ci, ci, ci, ip, ip, hp, hp, cf, cf, cu64, ci]
     lib.oracle_word2vecNegBf16.restype = None
     lib.oracle_word2vecEvalPosBf16.argtypes = [ci, ci, ci, ip, ip, ip, hp, hp, cd]
     lib.oracle_word2vecEvalPosBf16.restype = cd
@@ -159,14 +159,14 @@ class CPUMACH:
 
     # ---- bfloat16 tables (no counterpart in the reference; oracle/w2v_oracle_bf16.c) ---------
     @staticmethod
-    def word2vecPosBf16(nrows, ncols, skip, W, LB, UB, A, B, lrate, vexp, seed):
+    def word2vecPosBf16(nrows, ncols, skip, W, LB, UB, A, B, lrate, vexp, seed, hot_n=0):
         _load().oracle_word2vecPosBf16(nrows, ncols, skip, _i(W), _i(LB), _i(UB), _h(A), _h(B),
-                                       lrate, vexp, seed)
+                                       lrate, vexp, seed, hot_n)
 
     @staticmethod
-    def word2vecNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed):
+    def word2vecNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, hot_n=0):
         _load().oracle_word2vecNegBf16(nrows, ncols, nwa, nwb, _i(WA), _i(WB), _h(A), _h(B),
-                                       lrate, vexp, seed)
+                                       lrate, vexp, seed, hot_n)
 
     @staticmethod
     def word2vecEvalPosBf16(nrows, ncols, skip, W, LB, UB, A, B, floor=C_FLOOR):

@@ -16,7 +16,9 @@
  *   bf16 = (bits(x) + r16) >> 16                             (magnitude rounds up with
  *                                                             probability low16(x) / 65536)
  * slot names the write inside the unit: positive pass, context at offset j: (uint32)j, centre
- * column: 0; negative pass, B column k: k, A column j: 0x10000 + j.
+ * column: 0; negative pass, B column k: k, A column j: 0x10000 + j.  The columns of the first
+ * hot_n words go through an fp32 side buffer and are narrowed once, at the end of the call (see
+ * bf16_fold below), as the HIP library does for the words it treats as frequent.
  *
  * Parity pins (tests/test_oracle_bf16.py): the narrowing is checked for its two neighbours and
  * its mean (unbiased within sampling error) against numpy; on tables whose values are exactly
@@ -77,89 +79,148 @@ uint16_t oracle_bf16_narrow(float x, uint32_t key, uint32_t row) {
   return (uint16_t)((u + (bf16_fmix32(key ^ (row * 0x9E3779B9U)) >> 16)) >> 16);
 }
 
+/* Frequent words (ids below hot_n): during a call their columns are table + an fp32 side buffer;
+ * reads add the two in fp32, writes add the delta to the side buffer, and the end of the call
+ * narrows the sum back into the table with one rounding per element (unit 0xFFFFFFFF, slot
+ * (table << 31) | word; table 0 = A, 1 = B).  Elements whose side buffer is zero are left alone. */
+static float *bf16_side_alloc(int hot_n, int nrows) {
+  return (float *)calloc((size_t)(hot_n > 0 ? hot_n : 1) * nrows, sizeof(float));
+}
+
+static inline float bf16_read(const uint16_t *T, const float *side, int hot_n, int word,
+                              int64_t off, int nrows, int c) {
+  float v = bf16_widen(T[c + off]);
+  if (word < hot_n) v += side[(int64_t)word * nrows + c];
+  return v;
+}
+
+static void bf16_fold(uint16_t *T, float *side, int hot_n, int nrows, uint64_t seed, int table) {
+  int w, c;
+  for (w = 0; w < hot_n; w++) {
+    uint32_t key = oracle_bf16_key(seed, 0xFFFFFFFFU, ((uint32_t)table << 31) | (uint32_t)w);
+    for (c = 0; c < nrows; c++) {
+      float v = side[(int64_t)w * nrows + c];
+      if (v != 0.0f) {
+        int64_t at = (int64_t)w * nrows + c;
+        T[at] = oracle_bf16_narrow(bf16_widen(T[at]) + v, key, (uint32_t)c);
+      }
+    }
+  }
+}
+
 void oracle_word2vecPosBf16(int nrows, int ncols, int skip, const int *W, const int *LB,
                             const int *UB, uint16_t *A, uint16_t *B, float lrate, float vexp,
-                            uint64_t seed) {
-  int i, j, c, itmp;
+                            uint64_t seed, int hot_n) {
+  int i, j, c, wa, wb;
   int64_t ia, ib;
   float cv, ascale, bscale;
   float *daa = (float *)malloc((size_t)nrows * sizeof(float));
+  float *sa = bf16_side_alloc(hot_n, nrows), *sb = bf16_side_alloc(hot_n, nrows);
   (void)skip;
   for (i = 0; i < ncols; i++) {
-    itmp = W[i];
-    if (itmp < 0) continue;
-    ia = (int64_t)nrows * itmp;
-    ascale = pow(1 + itmp, vexp);
+    wa = W[i];
+    if (wa < 0) continue;
+    ia = (int64_t)nrows * wa;
+    ascale = pow(1 + wa, vexp);
     for (c = 0; c < nrows; c++) daa[c] = 0;
     for (j = LB[i]; j <= UB[i]; j++) {
       if (j != 0 && i + j >= 0 && i + j < ncols) {
-        itmp = W[i + j];
-        if (itmp >= 0) {
+        wb = W[i + j];
+        if (wb >= 0) {
           uint32_t key = oracle_bf16_key(seed, (uint32_t)i, (uint32_t)j);
-          ib = (int64_t)nrows * itmp;
-          bscale = pow(1 + itmp, vexp);
+          ib = (int64_t)nrows * wb;
+          bscale = pow(1 + wb, vexp);
           cv = 0;
-          for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+          for (c = 0; c < nrows; c++)
+            cv += bf16_read(A, sa, hot_n, wa, ia, nrows, c) * bf16_read(B, sb, hot_n, wb, ib, nrows, c);
           cv = bf16_oracle_sigmoid(cv);
           cv = lrate * (1.0f - cv);
           for (c = 0; c < nrows; c++) {
-            float a = bf16_widen(A[c + ia]), b = bf16_widen(B[c + ib]);
+            float a = bf16_read(A, sa, hot_n, wa, ia, nrows, c);
+            float b = bf16_read(B, sb, hot_n, wb, ib, nrows, c);
+            float db = bscale * cv * a;
             daa[c] += ascale * cv * b;
-            b += bscale * cv * a;
-            B[c + ib] = oracle_bf16_narrow(b, key, (uint32_t)c);
+            if (wb < hot_n)
+              sb[(int64_t)wb * nrows + c] += db;
+            else
+              B[c + ib] = oracle_bf16_narrow(b + db, key, (uint32_t)c);
           }
         }
       }
     }
     {
       uint32_t key = oracle_bf16_key(seed, (uint32_t)i, 0U);
-      for (c = 0; c < nrows; c++)
-        A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c], key, (uint32_t)c);
+      for (c = 0; c < nrows; c++) {
+        if (wa < hot_n)
+          sa[(int64_t)wa * nrows + c] += daa[c];
+        else
+          A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c], key, (uint32_t)c);
+      }
     }
   }
+  bf16_fold(A, sa, hot_n, nrows, seed, 0);
+  bf16_fold(B, sb, hot_n, nrows, seed, 1);
+  free(sb);
+  free(sa);
   free(daa);
 }
 
 void oracle_word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, const int *WA, const int *WB,
-                            uint16_t *A, uint16_t *B, float lrate, float vexp, uint64_t seed) {
-  int i, j, k, c, itmp;
+                            uint16_t *A, uint16_t *B, float lrate, float vexp, uint64_t seed,
+                            int hot_n) {
+  int i, j, k, c, wa, wb;
   int64_t ia, ib, ja;
   float cv, ascale, bscale;
   float *daa = (float *)malloc((size_t)(nwa > 0 ? nwa : 1) * nrows * sizeof(float));
   float *dbb = (float *)malloc((size_t)nrows * sizeof(float));
+  float *sa = bf16_side_alloc(hot_n, nrows), *sb = bf16_side_alloc(hot_n, nrows);
   for (i = 0; i < ncols; i++) {
     for (c = 0; c < nwa * nrows; c++) daa[c] = 0;
     for (k = 0; k < nwb; k++) {
       uint32_t key = oracle_bf16_key(seed, (uint32_t)i, (uint32_t)k);
-      itmp = WB[k + (int64_t)i * nwb];
-      ib = (int64_t)nrows * itmp;
-      bscale = pow(1 + itmp, vexp);
+      wb = WB[k + (int64_t)i * nwb];
+      ib = (int64_t)nrows * wb;
+      bscale = pow(1 + wb, vexp);
       for (c = 0; c < nrows; c++) dbb[c] = 0;
       for (j = 0; j < nwa; j++) {
-        itmp = WA[j + (int64_t)i * nwa];
-        ia = (int64_t)nrows * itmp;
-        ascale = pow(1 + itmp, vexp);
+        wa = WA[j + (int64_t)i * nwa];
+        ia = (int64_t)nrows * wa;
+        ascale = pow(1 + wa, vexp);
         cv = 0;
-        for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);
+        for (c = 0; c < nrows; c++)
+          cv += bf16_read(A, sa, hot_n, wa, ia, nrows, c) * bf16_read(B, sb, hot_n, wb, ib, nrows, c);
         cv = bf16_oracle_sigmoid(cv);
         cv = -lrate * cv;
         ja = (int64_t)j * nrows;
         for (c = 0; c < nrows; c++) {
-          dbb[c] += bscale * cv * bf16_widen(A[c + ia]);
-          daa[c + ja] += ascale * cv * bf16_widen(B[c + ib]);
+          dbb[c] += bscale * cv * bf16_read(A, sa, hot_n, wa, ia, nrows, c);
+          daa[c + ja] += ascale * cv * bf16_read(B, sb, hot_n, wb, ib, nrows, c);
         }
       }
-      for (c = 0; c < nrows; c++)
-        B[c + ib] = oracle_bf16_narrow(bf16_widen(B[c + ib]) + dbb[c], key, (uint32_t)c);
+      for (c = 0; c < nrows; c++) {
+        if (wb < hot_n)
+          sb[(int64_t)wb * nrows + c] += dbb[c];
+        else
+          B[c + ib] = oracle_bf16_narrow(bf16_widen(B[c + ib]) + dbb[c], key, (uint32_t)c);
+      }
     }
     for (j = 0; j < nwa; j++) {
       uint32_t key = oracle_bf16_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j);
       ja = (int64_t)j * nrows;
-      ia = (int64_t)nrows * WA[j + (int64_t)i * nwa];
-      for (c = 0; c < nrows; c++)
-        A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c + ja], key, (uint32_t)c);
+      wa = WA[j + (int64_t)i * nwa];
+      ia = (int64_t)nrows * wa;
+      for (c = 0; c < nrows; c++) {
+        if (wa < hot_n)
+          sa[(int64_t)wa * nrows + c] += daa[c + ja];
+        else
+          A[c + ia] = oracle_bf16_narrow(bf16_widen(A[c + ia]) + daa[c + ja], key, (uint32_t)c);
+      }
     }
   }
+  bf16_fold(A, sa, hot_n, nrows, seed, 0);
+  bf16_fold(B, sb, hot_n, nrows, seed, 1);
+  free(sb);
+  free(sa);
   free(dbb);
   free(daa);
 }

@@ -30,6 +30,18 @@ def gpu():
     return torch, CUMACH
 
 
+@pytest.fixture(params=[0, 1024, 4096])
+def hot(request):
+    """Number of frequent words the library routes through fp32 side buffers; the oracle is told
+    the same number."""
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    old = lib.w2v_get_bf16_hot_words()
+    assert lib.w2v_set_bf16_hot_words(request.param) == 0
+    yield request.param
+    lib.w2v_set_bf16_hot_words(old)
+
+
 def dev16(torch, h):
     """uint16 bit patterns -> device tensor of the same bits."""
     return torch.from_numpy(np.ascontiguousarray(h).view(np.int16)).cuda()
@@ -106,7 +118,7 @@ def test_eval_neg_bf16(gpu, oracle, d, V, G, nwa, nwb):
 @pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (512, 10, 100),
                                              (1, 2, 50), (65, 3, 100), (1280, 5, 40),
                                              (24, 40, 30), (130, 4, 100)])
-def test_pos_update_bf16(gpu, oracle, vexp, d, skip, ncentres):
+def test_pos_update_bf16(gpu, oracle, hot, vexp, d, skip, ncentres):
     torch, CUMACH = gpu
     rng = np.random.default_rng(d * 7 + skip)
     V = 20000
@@ -115,7 +127,7 @@ def test_pos_update_bf16(gpu, oracle, vexp, d, skip, ncentres):
     W[rng.random(W.shape[0]) < 0.05] = -1
     seed = 0x1234567 + d
     Ao, Bo = A.copy(), B.copy()
-    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, Ao, Bo, 0.025, vexp, seed)
+    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, Ao, Bo, 0.025, vexp, seed, hot)
     Ad, Bd = dev16(torch, A), dev16(torch, B)
     err = CUMACH.word2vecPosBf16(d, W.shape[0], skip, dev(torch, W), dev(torch, LB),
                                  dev(torch, UB), Ad, Bd, 0.025, vexp, seed)
@@ -129,7 +141,7 @@ def test_pos_update_bf16(gpu, oracle, vexp, d, skip, ncentres):
 @pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
                                          (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
                                          (40, 70, 3, 40), (300, 6, 2, 100), (130, 4, 6, 100)])
-def test_neg_update_bf16(gpu, oracle, vexp, d, nwa, nwb, G):
+def test_neg_update_bf16(gpu, oracle, hot, vexp, d, nwa, nwb, G):
     torch, CUMACH = gpu
     rng = np.random.default_rng(d * 5 + nwa)
     V = 20000
@@ -137,7 +149,7 @@ def test_neg_update_bf16(gpu, oracle, vexp, d, nwa, nwb, G):
     WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
     seed = 0x7654321 + d
     Ao, Bo = A.copy(), B.copy()
-    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.025, vexp, seed)
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.025, vexp, seed, hot)
     Ad, Bd = dev16(torch, A), dev16(torch, B)
     err = CUMACH.word2vecNegBf16(d, G, nwa, nwb, dev(torch, WA), dev(torch, WB), Ad, Bd, 0.025,
                                  vexp, seed)
@@ -179,7 +191,7 @@ def test_updates_within_1e_4_of_the_fp32_oracle_at_initial_scale(gpu, oracle):
     assert np.abs(Aw - cpumach.bf16_widen(A)).max() > 10 * UPDATE_ATOL
 
 
-def test_unaligned_tables_take_the_halfword_path(gpu, oracle):
+def test_unaligned_tables_take_the_halfword_path(gpu, oracle, hot):
     # an even d with a table that starts on an odd halfword: columns are 2-byte aligned only
     torch, CUMACH = gpu
     d, V, G, nwa, nwb = 64, 3000, 100, 5, 5
@@ -187,7 +199,7 @@ def test_unaligned_tables_take_the_halfword_path(gpu, oracle):
     A, B = tables16(rng, V, d, 0.2)
     WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
     Ao, Bo = A.copy(), B.copy()
-    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.025, 0.0, 3)
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.025, 0.0, 3, hot)
     buf_a = torch.zeros(V * d + 1, dtype=torch.int16, device="cuda")
     buf_b = torch.zeros(V * d + 1, dtype=torch.int16, device="cuda")
     Ad, Bd = buf_a[1:], buf_b[1:]
@@ -229,6 +241,10 @@ def test_empty_and_rejected_arguments_bf16(gpu):
     assert CUMACH.word2vecPosBf16(1281, 1, 5, i, i, i, t, t, 0.1, 0.0, 1) == 1
     assert CUMACH.word2vecPosBf16(8, 1, 5, None, i, i, t, t, 0.1, 0.0, 1) == 1
     assert CUMACH.word2vecNegBf16(8, 1, 2, 9, i, i, t, t, 0.1, 0.0, 1) == 1
+    from bidmach_amd.cumach import load_library
+    assert load_library().w2v_set_bf16_hot_words(-1) == 1
+    assert load_library().w2v_set_bf16_hot_words(4097) == 1
+    assert load_library().w2v_get_bf16_hot_words() == 1024
     assert CUMACH.word2vecEvalPosBf16(8, 1, 5, i, i, i, t, t, None) == 1
     assert CUMACH.word2vecEvalNegBf16(8, 1, 2, 2, i, i, t, None, r) == 1
     assert (t == 0).all()
@@ -240,7 +256,8 @@ def test_empty_and_rejected_arguments_bf16(gpu):
 # 1.35746 on this stream, the sequential fp32 oracle 1.35746 as well).
 # ---------------------------------------------------------------------------------------------
 
-def test_heldout_loss_next_to_the_fp32_operators():
+@pytest.mark.parametrize("hot_words", [1024, 0])
+def test_heldout_loss_next_to_the_fp32_operators(hot_words):
     import torch
     from bidmach_amd.cumach import CUMACH, check, f32_to_bf16
     V, D, N, SKIP, NNEG, NREUSE, NMB, LR0 = 10000, 100, 100000, 5, 5, 5, 30, 0.025
@@ -256,6 +273,8 @@ def test_heldout_loss_next_to_the_fp32_operators():
         return [torch.from_numpy(x).cuda() for x in (W, LB, UB, WA, WB)] + [G]
 
     stream = [minibatch(i) for i in range(NMB + 1)]
+    from bidmach_amd.cumach import load_library
+    assert load_library().w2v_set_bf16_hot_words(hot_words) == 0
     Bh, Ah = corpus.init_tables(V, D, 42)
     A32, B32 = torch.from_numpy(Ah).cuda(), torch.from_numpy(Bh).cuda()
     A16 = torch.zeros(V * D, dtype=torch.int16, device="cuda")
@@ -277,10 +296,12 @@ def test_heldout_loss_next_to_the_fp32_operators():
     check(CUMACH.word2vecEvalPosBf16(D, N, SKIP, W, LB, UB, A16, B16, r[2:3]), "epos16")
     check(CUMACH.word2vecEvalNegBf16(D, G, NNEG, NREUSE, WA, WB, A16, B16, r[3:4]), "eneg16")
     r = r.cpu().numpy()
+    load_library().w2v_set_bf16_hot_words(1024)
     loss32 = -(r[0] + r[1] / NNEG) / (G * NREUSE)
     loss16 = -(r[2] + r[3] / NNEG) / (G * NREUSE)
-    print("\nheld-out loss after %d minibatches: fp32 tables %.5f, bf16 tables %.5f (%+.2f%%)"
-          % (NMB, loss32, loss16, 100.0 * (loss16 / loss32 - 1.0)))
+    print("\nheld-out loss after %d minibatches: fp32 tables %.5f, bf16 tables (%d frequent words "
+          "through side buffers) %.5f (%+.2f%%)"
+          % (NMB, loss32, hot_words, loss16, 100.0 * (loss16 / loss32 - 1.0)))
     assert np.isfinite(loss16)
     assert loss16 < 1.386                        # better than the untrained model
     assert abs(loss16 - loss32) <= 0.005 * loss32

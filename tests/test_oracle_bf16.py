@@ -87,9 +87,10 @@ def test_eval_equals_fp32_oracle_on_widened_tables(oracle, d, V, N, skip):
         oracle.word2vecEvalNeg(d, G, nwa, nwb, WA, WB, A32, B32, 1)
 
 
+@pytest.mark.parametrize("hot", [0, 1500])
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
 @pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 60), (33, 3, 40), (1, 2, 20)])
-def test_pos_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, skip, ncentres):
+def test_pos_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, skip, ncentres, hot):
     # collision-free: every column is written once, so every stored element must be one of the
     # two bf16 neighbours of what the fp32 oracle computes from the widened tables
     rng = np.random.default_rng(d + skip)
@@ -100,7 +101,7 @@ def test_pos_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, skip, ncen
     A32, B32 = cpumach.bf16_widen(A).copy(), cpumach.bf16_widen(B).copy()
     oracle.word2vecPos(d, W.shape[0], skip, W, LB, UB, A32, B32, 0.025, vexp, 1)
     A16, B16 = A.copy(), B.copy()
-    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A16, B16, 0.025, vexp, 11)
+    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A16, B16, 0.025, vexp, 11, hot)
     assert neighbours_ok(A16, A32) and neighbours_ok(B16, B32)
     changed = (A16 != A).any(axis=1).sum() + (B16 != B).any(axis=1).sum()
     assert changed > ncentres
@@ -109,17 +110,18 @@ def test_pos_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, skip, ncen
     assert (A16[untouched] == A[untouched]).all() and (B16[untouched] == B[untouched]).all()
     # same seed, same bits; another seed, other roundings
     A2, B2 = A.copy(), B.copy()
-    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A2, B2, 0.025, vexp, 11)
+    oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A2, B2, 0.025, vexp, 11, hot)
     assert (A2 == A16).all() and (B2 == B16).all()
     if d > 1:
-        oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A2, B2, 0.025, vexp, 12)
+        oracle.word2vecPosBf16(d, W.shape[0], skip, W, LB, UB, A2, B2, 0.025, vexp, 12, hot)
         assert (B2 != B16).any()
 
 
+@pytest.mark.parametrize("hot", [0, 1500])
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
 @pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 60), (33, 7, 8, 30), (1, 1, 1, 20),
                                          (20, 15, 3, 20)])
-def test_neg_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, nwa, nwb, G):
+def test_neg_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, nwa, nwb, G, hot):
     rng = np.random.default_rng(d + nwa)
     V = 4000
     A, B = tables16(rng, V, d, 0.5 / d ** 0.25)
@@ -127,7 +129,7 @@ def test_neg_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, nwa, nwb, 
     A32, B32 = cpumach.bf16_widen(A).copy(), cpumach.bf16_widen(B).copy()
     oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, A32, B32, 0.025, vexp, 1)
     A16, B16 = A.copy(), B.copy()
-    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, A16, B16, 0.025, vexp, 5)
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, A16, B16, 0.025, vexp, 5, hot)
     assert neighbours_ok(A16, A32) and neighbours_ok(B16, B32)
     assert (A16 != A).any() and (B16 != B).any()
 
@@ -152,3 +154,40 @@ def test_mean_over_seeds_approaches_the_fp32_result(oracle):
     err = np.abs(accA[rows] / nseed - A32[rows])
     assert (err <= 5 * step / np.sqrt(nseed) + 1e-12).all()
     assert np.abs(cpumach.bf16_widen(A16)[rows] - A32[rows]).max() > err.max()
+
+
+def test_side_buffers_follow_the_sequential_fp32_run_on_colliding_minibatches(oracle):
+    # with every word routed through the fp32 side buffers nothing is rounded to bf16 inside a
+    # call, so even on a Zipf minibatch, where later units read what earlier ones wrote, the
+    # result is the sequential fp32 oracle's (on the widened tables) narrowed once: within one
+    # bf16 step, plus a few fp32 ulps for the different association of the sums
+    rng = np.random.default_rng(21)
+    d, V, N, skip, nwa, nwb = 24, 300, 3000, 4, 5, 4
+    A, B = tables16(rng, V, d, 0.3)
+    W = corpus.zipf_stream(N, V, 1.0, seed=4)
+    W[rng.random(N) < 0.05] = -1
+    LB, UB = corpus.window_bounds(N, skip, rng)
+    G = 400
+    WA = rng.integers(0, V, G * nwa).astype(np.int32)
+    WB = corpus.zipf_stream(G * nwb, V, 1.0, seed=5)
+
+    def close(got16, want32):
+        step = np.abs(want32) * 2.0 ** -7
+        slack = np.abs(want32).max() * 2.0 ** -17
+        return bool((np.abs(cpumach.bf16_widen(got16) - want32) <= step + slack).all())
+
+    A32, B32 = cpumach.bf16_widen(A).copy(), cpumach.bf16_widen(B).copy()
+    oracle.word2vecPos(d, N, skip, W, LB, UB, A32, B32, 0.025, 0.5, 1)
+    A16, B16 = A.copy(), B.copy()
+    oracle.word2vecPosBf16(d, N, skip, W, LB, UB, A16, B16, 0.025, 0.5, 8, V)
+    assert close(A16, A32) and close(B16, B32)
+    assert np.abs(A32 - cpumach.bf16_widen(A)).max() > 0.05      # many updates piled up
+
+    A32, B32 = cpumach.bf16_widen(A).copy(), cpumach.bf16_widen(B).copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, A32, B32, 0.025, 0.5, 1)
+    A16, B16 = A.copy(), B.copy()
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, A16, B16, 0.025, 0.5, 9, V)
+    assert close(A16, A32) and close(B16, B32)
+    # words the call never touched keep their bits
+    untouched = np.setdiff1d(np.arange(V), np.concatenate([WA, WB]))
+    assert (A16[untouched] == A[untouched]).all() and (B16[untouched] == B[untouched]).all()
