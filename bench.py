@@ -158,6 +158,12 @@ def main():
     ap.add_argument("--hot-mode", type=int, default=-1, choices=[-1, 0, 1, 2],
                     help="w2v_set_hot_update_mode: -1 the library's per-launch choice (default), "
                          "0 exact shadow copies, 1 combining shadow copies, 2 no shadow copies")
+    ap.add_argument("--bf16-hot-words", type=int, default=-1,
+                    help="bf16 workload: w2v_set_bf16_hot_words (frequent words updated through "
+                         "fp32 side buffers); -1 = the library's default")
+    ap.add_argument("--max-workgroups", type=int, default=0,
+                    help="w2v_set_max_workgroups: bound on the workgroups of the update kernels "
+                         "(0 = the whole device)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -178,6 +184,10 @@ def main():
     from bidmach_amd.cumach import load_library
     load_library().w2v_set_hot_update_mode(args.hot_mode)
     load_library().w2v_set_rare_update_mode(args.rare_mode)
+    if args.bf16_hot_words >= 0:
+        check(load_library().w2v_set_bf16_hot_words(args.bf16_hot_words), "w2v_set_bf16_hot_words")
+    if args.max_workgroups > 0:
+        load_library().w2v_set_max_workgroups(args.max_workgroups)
     cfg = dict(WORKLOADS[args.workload])
     if args.tokens > 0:
         cfg["tokens"] = args.tokens
@@ -353,8 +363,11 @@ def main():
     if evaluating:
         out["config"]["mode"] = "eval"
         out["roofline"]["traffic"] = None
+    if args.max_workgroups > 0:
+        out["config"]["max_workgroups"] = args.max_workgroups
     if bf16:
         out["config"]["storage"] = "bf16"
+        out["config"]["hot_words"] = load_library().w2v_get_bf16_hot_words()
         out["config"]["operators"] = "word2vecPosBf16+word2vecNegBf16"
     if args.hot_mode != -1:
         out["config"]["hot_update_mode"] = args.hot_mode

@@ -104,44 +104,76 @@ __device__ __forceinline__ uint32_t cas_word(uint32_t* p, uint32_t expected, uin
 // the column as this wave read it (the first guess; the exchange fails and is repeated with the
 // value found if the column has changed since).  The random bits depend on (key, row) only, so a
 // repeated attempt rounds the same way.
+// First round of the exchange for a column of 4-byte words: the words are issued and their
+// results left in `found`, not waited for, so that a caller can put the exchanges of several
+// columns (or a load it will need next) in flight before the first result is looked at.
+template <int RP>
+__device__ __forceinline__ void cas_first(uint16_t* col, const float (&seen)[2 * RP],
+                                          const float (&delta)[2 * RP], int lane, int d,
+                                          uint32_t key, uint32_t (&guess)[RP],
+                                          uint32_t (&found)[RP]) {
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    const int e = r * 128 + 2 * lane;
+    guess[r] = (__builtin_bit_cast(uint32_t, seen[2 * r]) >> 16) |
+               (__builtin_bit_cast(uint32_t, seen[2 * r + 1]) & 0xFFFF0000U);
+    found[r] = guess[r];
+    if (e < d) {
+      const float lo = seen[2 * r] + delta[2 * r];
+      const float hi = seen[2 * r + 1] + delta[2 * r + 1];
+      const uint32_t want = sr_narrow(lo, key, (uint32_t)e) |
+                            (sr_narrow(hi, key, (uint32_t)(e + 1)) << 16);
+      found[r] = cas_word(reinterpret_cast<uint32_t*>(col + e), guess[r], want);
+    }
+  }
+}
+
+// Looks at the results of cas_first and repeats the words that found another value, with that
+// value as the new guess, until every word has been exchanged.
+template <int RP>
+__device__ __forceinline__ void cas_rest(uint16_t* col, const float (&delta)[2 * RP], int lane,
+                                         int d, uint32_t key, uint32_t (&guess)[RP],
+                                         uint32_t (&found)[RP]) {
+  bool open[RP];
+  bool any = false;
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    open[r] = found[r] != guess[r];   // words beyond d were never issued: found == guess
+    guess[r] = found[r];
+    any = any || open[r];
+  }
+  while (any) {
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      if (open[r]) {
+        const int e = r * 128 + 2 * lane;
+        const float lo = __builtin_bit_cast(float, guess[r] << 16) + delta[2 * r];
+        const float hi = __builtin_bit_cast(float, guess[r] & 0xFFFF0000U) + delta[2 * r + 1];
+        const uint32_t want = sr_narrow(lo, key, (uint32_t)e) |
+                              (sr_narrow(hi, key, (uint32_t)(e + 1)) << 16);
+        found[r] = cas_word(reinterpret_cast<uint32_t*>(col + e), guess[r], want);
+      }
+    }
+    any = false;
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      if (open[r]) {
+        open[r] = found[r] != guess[r];
+        guess[r] = found[r];
+        any = any || open[r];
+      }
+    }
+  }
+}
+
 template <int RP, bool ALIGNED>
 __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 * RP],
                                           const float (&delta)[2 * RP], int lane, int d,
                                           uint32_t key) {
   if (ALIGNED) {
     uint32_t guess[RP], found[RP];
-    bool open[RP];
-#pragma unroll
-    for (int r = 0; r < RP; ++r) {
-      guess[r] = (__builtin_bit_cast(uint32_t, seen[2 * r]) >> 16) |
-                 (__builtin_bit_cast(uint32_t, seen[2 * r + 1]) & 0xFFFF0000U);
-      found[r] = guess[r];
-      open[r] = r * 128 + 2 * lane < d;
-    }
-    bool any = true;
-    while (any) {
-      // all of the lane's words are in flight together; only the ones that failed go again
-#pragma unroll
-      for (int r = 0; r < RP; ++r) {
-        if (open[r]) {
-          const int e = r * 128 + 2 * lane;
-          const float lo = __builtin_bit_cast(float, guess[r] << 16) + delta[2 * r];
-          const float hi = __builtin_bit_cast(float, guess[r] & 0xFFFF0000U) + delta[2 * r + 1];
-          const uint32_t want = sr_narrow(lo, key, (uint32_t)e) |
-                                (sr_narrow(hi, key, (uint32_t)(e + 1)) << 16);
-          found[r] = cas_word(reinterpret_cast<uint32_t*>(col + e), guess[r], want);
-        }
-      }
-      any = false;
-#pragma unroll
-      for (int r = 0; r < RP; ++r) {
-        if (open[r]) {
-          open[r] = found[r] != guess[r];
-          guess[r] = found[r];
-          any = any || open[r];
-        }
-      }
-    }
+    cas_first<RP>(col, seen, delta, lane, d, key, guess, found);
+    cas_rest<RP>(col, delta, lane, d, key, guess, found);
   } else {
     // columns on 2-byte boundaries: each element is exchanged inside the aligned word that
     // holds it, the other half of the word being written back as found

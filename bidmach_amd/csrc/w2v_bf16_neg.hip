@@ -53,13 +53,25 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) dbb[k][r] = 0.0f;
     }
+    // the next A column is requested before the current one is written back, so its gather
+    // overlaps the exchange; a word that occurs twice among a group's A words is then dotted as
+    // it was before the first of its two updates, as in the reference, which writes A after
+    // every dot of the group
+    float a[2 * RP], anext[2 * RP];
+    int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa]);
+    load_col16<RP, ALIGNED, !EVAL>(a, A + (int64_t)wa * d, lane, d);
+    if (!EVAL && wa < hot.n) add_side_col<RP>(a, hot.sa + (int64_t)wa * d, lane, d);
     for (int j = 0; j < nwa; ++j) {
-      const int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa + j]);
       uint16_t* acol = A + (int64_t)wa * d;
-      float a[2 * RP], daa[2 * RP];
-      load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
       const bool ahot = !EVAL && wa < hot.n;
-      if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)wa * d, lane, d);
+      int wanext = 0;
+      if (j + 1 < nwa) {
+        wanext = __builtin_amdgcn_readfirstlane(WA[i * nwa + j + 1]);
+        load_col16<RP, ALIGNED, !EVAL>(anext, A + (int64_t)wanext * d, lane, d);
+        if (!EVAL && wanext < hot.n)
+          add_side_col<RP>(anext, hot.sa + (int64_t)wanext * d, lane, d);
+      }
+      float daa[2 * RP];
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
       const float ascale = EVAL ? 1.0f : scale_of(wa, vexp, smode);
@@ -91,16 +103,42 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
           add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
                                  sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
       }
+      if (j + 1 < nwa) {
+        wa = wanext;
+#pragma unroll
+        for (int r = 0; r < 2 * RP; ++r) a[r] = anext[r];
+      }
     }
     if (!EVAL) {
+      if (ALIGNED) {
+        // the exchanges of all B columns are in flight together before the first result is used
+        uint32_t guess[MAXB][RP], found[MAXB][RP];
 #pragma unroll
-      for (int k = 0; k < MAXB; ++k) {
-        if (k < nwb) {
-          if (wb[k] < hot.n)
-            atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
-          else
-            add_col16<RP, ALIGNED>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
+        for (int k = 0; k < MAXB; ++k) {
+          if (k < nwb) {
+            if (wb[k] < hot.n)
+              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
+            else
+              cas_first<RP>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
+                            sr_key(seed, (uint32_t)i, (uint32_t)k), guess[k], found[k]);
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < MAXB; ++k) {
+          if (k < nwb && wb[k] >= hot.n)
+            cas_rest<RP>(B + (int64_t)wb[k] * d, dbb[k], lane, d,
+                         sr_key(seed, (uint32_t)i, (uint32_t)k), guess[k], found[k]);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < MAXB; ++k) {
+          if (k < nwb) {
+            if (wb[k] < hot.n)
+              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
+            else
+              add_col16<RP, false>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
                                    sr_key(seed, (uint32_t)i, (uint32_t)k));
+          }
         }
       }
     }

@@ -48,16 +48,38 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
-    for (int j = lb; j <= ub; ++j) {
-      const int64_t p = i + j;
-      if (j == 0 || p < 0 || p >= n) continue;
-      const int wb = __builtin_amdgcn_readfirstlane(W[p]);
-      if (wb < 0) continue;
+    // window clipped to the minibatch, so that the scan below stays inside W
+    const int lo = lb < -i ? (int)-i : lb;
+    const int hi = ub > n - 1 - i ? (int)(n - 1 - i) : ub;
+    // next valid context at or after offset j0 (hi + 1 if none); its word id goes to `word`
+    auto next_context = [&](int j0, int& word) {
+      for (int j = j0; j <= hi; ++j) {
+        if (j == 0) continue;
+        const int x = __builtin_amdgcn_readfirstlane(W[i + j]);
+        if (x >= 0) {
+          word = x;
+          return j;
+        }
+      }
+      return hi + 1;
+    };
+    auto load_b = [&](float (&x)[2 * RP], int word) {
+      load_col16<RP, ALIGNED, !EVAL>(x, B + (int64_t)word * d, lane, d);
+      if (!EVAL && word < hot.n) add_side_col<RP>(x, hot.sb + (int64_t)word * d, lane, d);
+    };
+    int wb = 0;
+    int j = next_context(lo, wb);
+    float b[2 * RP], bnext[2 * RP];
+    if (j <= hi) load_b(b, wb);
+    while (j <= hi) {
+      // the next context's column is requested before this one is written back, so its gather
+      // overlaps the exchange -- unless it is the same word again, which has to see this update
+      int wbnext = 0;
+      const int jnext = next_context(j + 1, wbnext);
+      const bool ahead = jnext <= hi && wbnext != wb;
+      if (ahead) load_b(bnext, wbnext);
       uint16_t* bcol = B + (int64_t)wb * d;
-      float b[2 * RP];
-      load_col16<RP, ALIGNED, !EVAL>(b, bcol, lane, d);
       const bool bhot = !EVAL && wb < hot.n;
-      if (bhot) add_side_col<RP>(b, hot.sb + (int64_t)wb * d, lane, d);
       float part = 0.0f;
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[r], part);
@@ -79,6 +101,11 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
         else
           add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
+      if (jnext <= hi && !ahead) load_b(bnext, wbnext);
+#pragma unroll
+      for (int r = 0; r < 2 * RP; ++r) b[r] = bnext[r];
+      j = jnext;
+      wb = wbnext;
     }
     if (!EVAL) {
       if (ahot)

@@ -65,6 +65,10 @@ class Options:
         self.dualMode = False
         self.doHead = 1
         self.deviceWordMats = True   # build the index arrays on the GPU when the model is on one
+        # element type of the model on the device: "fp32" (the reference's), or "bf16" (no
+        # counterpart in the reference: fp32 arithmetic, stochastic-rounded write-back, half the
+        # memory; single-table models only)
+        self.storage = "fp32"
         for k, v in kw.items():
             if not hasattr(self, k):
                 raise AttributeError("unknown Word2Vec option %r" % k)
@@ -114,6 +118,19 @@ class Word2Vec:
         # (columns, dim) C-order == dim x columns column-major, the layout the operators take
         self.modelmats = [torch.from_numpy(np.ascontiguousarray(m)).to(self.device)
                           for m in modelmats]
+        if o.storage == "bf16":
+            if self._sliced():
+                raise ValueError("bf16 storage takes a single-table model (nSlices = 1, one part)")
+            from .cumach import f32_to_bf16
+            narrow = []
+            for m in self.modelmats:
+                h = torch.empty(m.shape, dtype=torch.bfloat16, device=self.device)
+                f32_to_bf16(m.numel(), m, h)
+                narrow.append(h)
+            self.modelmats = narrow
+        elif o.storage != "fp32":
+            raise ValueError("unknown storage %r" % (o.storage,))
+        self._seed16 = 0
         self.expt = 1.0 / (1.0 - o.wexpt)
         self.salpha = o.wsample * math.log(o.vocabSize)
         self._ret = torch.zeros(2, dtype=torch.float32, device=self.device)
@@ -238,13 +255,28 @@ class Word2Vec:
     # them.
     def procPositives(self, nskip, words, lb, ub, model1, model2, lrate, vexp):
         nrows = model1.shape[1]
+        if self.opts.storage == "bf16":
+            check(CUMACH.word2vecPosBf16(nrows, words.shape[0], nskip, words, lb, ub, model1,
+                                         model2, lrate, vexp, self._next_seed16()),
+                  "word2vecPosBf16")
+            return
         check(CUMACH.word2vecPosAsync(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
                                       lrate, vexp), "word2vecPos")
 
     def procNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb, lrate, vexp):
         nrows = modela.shape[1]
+        if self.opts.storage == "bf16":
+            check(CUMACH.word2vecNegBf16(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
+                                         modela, modelb, lrate, vexp, self._next_seed16()),
+                  "word2vecNegBf16")
+            return
         check(CUMACH.word2vecNegAsync(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
                                       modela, modelb, lrate, vexp), "word2vecNeg")
+
+    def _next_seed16(self):
+        """A new key for the stochastic rounding of every bf16 update call."""
+        self._seed16 += 1
+        return ((int(self.opts.seed) & 0xFFFFFFFF) << 32) | (self._seed16 & 0xFFFFFFFF)
 
     def synchronize(self):
         """Waits for the enqueued updates and raises if any of them failed."""
@@ -253,6 +285,11 @@ class Word2Vec:
 
     def evalPositives(self, nskip, words, lb, ub, model1, model2):
         nrows = model1.shape[1]
+        if self.opts.storage == "bf16":
+            self._ret64[0:1].zero_()
+            check(CUMACH.word2vecEvalPosBf16(nrows, words.shape[0], nskip, words, lb, ub, model1,
+                                             model2, self._ret64[0:1]), "word2vecEvalPosBf16")
+            return float(self._ret64[0].item())
         self._ret[0:1].zero_()                                  # retEvalPos.clear (:476)
         check(CUMACH.word2vecEvalPos(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
                                      self._ret[0:1]), "word2vecEvalPos")
@@ -260,6 +297,12 @@ class Word2Vec:
 
     def evalNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb):
         nrows = modela.shape[1]
+        if self.opts.storage == "bf16":
+            self._ret64[1:2].zero_()
+            check(CUMACH.word2vecEvalNegBf16(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa,
+                                             wordsb, modela, modelb, self._ret64[1:2]),
+                  "word2vecEvalNegBf16")
+            return float(self._ret64[1].item())
         self._ret[1:2].zero_()
         check(CUMACH.word2vecEvalNeg(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
                                      modela, modelb, self._ret[1:2]), "word2vecEvalNeg")
@@ -349,7 +392,8 @@ class Word2Vec:
         with open(fname + "options.json", "w") as f:
             json.dump({k: v for k, v in vars(self.opts).items()}, f, indent=1, sort_keys=True)
         for i, m in enumerate(self.modelmats):
-            matio.saveMat(fname + "modelmat%02d.lz4" % i, m.cpu().numpy().T)
+            # a bf16 model is written widened: the files hold fp32, as the reference's do
+            matio.saveMat(fname + "modelmat%02d.lz4" % i, m.float().cpu().numpy().T)
 
     def load(self, fname, useJson=True):
         """Reads the model matrices `fname + "modelmat%02d.lz4"` (as many as exist) and, with

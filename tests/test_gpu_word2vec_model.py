@@ -211,3 +211,38 @@ def test_train_from_word_file_then_checkpoint_round_trip(tmp_path):
     s1 = m.evalbatch(held, 0, 4000)
     s2 = m2.evalbatch(held, 0, 4000)
     assert s1 < -0.1 and s1 == s2
+
+
+def test_bf16_storage_trains_like_fp32_and_round_trips_through_a_checkpoint(tmp_path):
+    """The same training loop on a bfloat16 model (no counterpart in the reference): scores
+    follow the fp32 model's, and a checkpoint written from it (widened to fp32 files) loads back
+    into an identical bf16 model."""
+    import os
+    import torch
+    stream = make_stream(4000 * 9, 3000, seed=8)
+    scores = {}
+    models = {}
+    for storage in ("fp32", "bf16"):
+        o = Options(vocabSize=3000, dim=32, batchSize=4000, lrate=0.05, evalStep=3, seed=5,
+                    storage=storage)
+        m = Word2Vec(o)
+        res = m.train(stream, npasses=2)
+        assert len(res) == 8
+        scores[storage] = [r[1] for r in res]
+        models[storage] = m
+    assert models["bf16"].modelmats[0].dtype == torch.bfloat16
+    assert all(np.isfinite(s) and s < 0 for s in scores["bf16"])
+    assert scores["bf16"][-1] > scores["bf16"][0]
+    # both runs see the same minibatches; the scores differ by rounding noise only
+    for a, b in zip(scores["fp32"], scores["bf16"]):
+        assert b == pytest.approx(a, rel=0.01)
+    m = models["bf16"]
+    prefix = str(tmp_path / "model16") + os.sep
+    m.save(prefix)
+    m2 = Word2Vec(Options(dim=32, batchSize=4000))
+    m2.load(prefix)
+    assert m2.opts.storage == "bf16"
+    for a, b in zip(m.modelmats, m2.modelmats):
+        assert b.dtype == torch.bfloat16 and bool((a.view(torch.int16) == b.view(torch.int16)).all())
+    with pytest.raises(ValueError):
+        Word2Vec(Options(vocabSize=3000, dim=32, nSlices=2, storage="bf16")).init(4000)
