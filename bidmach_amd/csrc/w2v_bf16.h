@@ -60,31 +60,34 @@ __device__ __forceinline__ uint32_t sr_narrow(float x, uint32_t key, uint32_t ro
   return (u + (sr_fmix32(key ^ (row * 0x9E3779B9U)) >> 16)) >> 16;
 }
 
-// Loads of the update kernels are device-scope (relaxed atomic loads): a plain
-// load may be served from the CU's own L1 or the XCD's own L2, which other CUs' and XCDs' stores
-// do not reach, so a wave that meets a frequent word again would read the column as it was the
-// first time and write back a sum that drops everything the rest of the device added since.
-// The forward kernels, which only read, use plain loads (DEVICE_SCOPE = false).
-template <bool DEVICE_SCOPE, typename T>
-__device__ __forceinline__ T load_elt(const T* p) {
-  if (DEVICE_SCOPE) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// A plain load may be served from the CU's own L1 or the XCD's own L2, which other CUs' and XCDs'
+// writes do not reach: a column that stays resident there is read as it was the first time.  The
+// columns of the frequent words do stay resident, so they (and their side buffers) are read with
+// device-scope loads (`fresh`); with plain loads and plain stores a frequent column ended as
+// whichever wave wrote last had left it.  Every other column is read with a plain load, like the
+// fp32 kernels': its line lives in an L2 for tens of microseconds at most, and the write-back does
+// not trust what was read -- the exchange compares against memory and repeats with the value
+// found.
+template <typename T>
+__device__ __forceinline__ T load_elt(const T* p, bool fresh) {
+  if (fresh) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return *p;
 }
 
-template <int RP, bool ALIGNED, bool DEVICE_SCOPE>
+template <int RP, bool ALIGNED>
 __device__ __forceinline__ void load_col16(float (&x)[2 * RP], const uint16_t* col, int lane,
-                                           int d) {
+                                           int d, bool fresh) {
 #pragma unroll
   for (int r = 0; r < RP; ++r) {
     const int e = r * 128 + 2 * lane;
     if (ALIGNED) {
       uint32_t v = 0;
-      if (e < d) v = load_elt<DEVICE_SCOPE>(reinterpret_cast<const uint32_t*>(col + e));
+      if (e < d) v = load_elt(reinterpret_cast<const uint32_t*>(col + e), fresh);
       x[2 * r] = __builtin_bit_cast(float, v << 16);
       x[2 * r + 1] = __builtin_bit_cast(float, v & 0xFFFF0000U);
     } else {
-      const uint32_t lo = (e < d) ? load_elt<DEVICE_SCOPE>(col + e) : 0U;
-      const uint32_t hi = (e + 1 < d) ? load_elt<DEVICE_SCOPE>(col + e + 1) : 0U;
+      const uint32_t lo = (e < d) ? load_elt(col + e, fresh) : 0U;
+      const uint32_t hi = (e + 1 < d) ? load_elt(col + e + 1, fresh) : 0U;
       x[2 * r] = __builtin_bit_cast(float, lo << 16);
       x[2 * r + 1] = __builtin_bit_cast(float, hi << 16);
     }
@@ -184,7 +187,7 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
         const uintptr_t addr = reinterpret_cast<uintptr_t>(col + e);
         uint32_t* word = reinterpret_cast<uint32_t*>(addr & ~(uintptr_t)3);
         const int shift = (addr & 2) ? 16 : 0;
-        uint32_t guess = load_elt<true>(word);
+        uint32_t guess = load_elt(word, true);
         for (;;) {
           const float x = __builtin_bit_cast(float, ((guess >> shift) & 0xFFFFU) << 16) + delta[r];
           const uint32_t want = (guess & ~(0xFFFFU << shift)) |
@@ -201,7 +204,7 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
 // Frequent words.  Word ids are frequency ranks, so the first few hundred ids take most of the
 // updates of a call, and a compare-and-swap on a column that thousands of waves update at once
 // fails nearly every time.  The columns of the words below `n` therefore have an fp32 side
-// buffer each (sa for table A, sb for table B; n x d floats, zero between calls): while a call
+// buffer each (sa for table A, sb for table B; n x side_stride(d) floats, zero between calls): while a call
 // runs, the value of such a column is widen(table) + side buffer, readers add the two in fp32,
 // and writers add their delta to the side buffer with float atomics, which need no retry.  A small
 // kernel at the end of the call narrows table + side buffer back into the table (one stochastic
@@ -212,13 +215,23 @@ struct HotCols {
   int n;
 };
 
+// Inside a side buffer a column is stored in the order the wave holds it: the lane's first
+// elements of a round, then its second ones (element 128 r + 2 l + h sits at 128 r + 64 h + l),
+// padded to whole rounds.  A float-atomic instruction of the wave then covers 64 consecutive
+// floats, two whole cache lines, and an update touches every line of the column once; in element
+// order it would touch every line twice, and the updates of the most frequent word, which retire
+// one after the other on each of its lines, are the critical path of a call.
+__host__ __device__ __forceinline__ int side_stride(int d) { return (d + 127) / 128 * 128; }
+
 template <int RP>
 __device__ __forceinline__ void add_side_col(float (&x)[2 * RP], const float* side, int lane,
                                              int d) {
 #pragma unroll
   for (int r = 0; r < 2 * RP; ++r) {
     const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
-    if (e < d) x[r] += __hip_atomic_load(side + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (e < d)
+      x[r] += __hip_atomic_load(side + (r >> 1) * 128 + (r & 1) * 64 + lane, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -228,7 +241,7 @@ __device__ __forceinline__ void atomic_add_side_col(float* side, const float (&d
 #pragma unroll
   for (int r = 0; r < 2 * RP; ++r) {
     const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
-    if (e < d) atomicAdd(side + e, delta[r]);
+    if (e < d) atomicAdd(side + (r >> 1) * 128 + (r & 1) * 64 + lane, delta[r]);
   }
 }
 
@@ -239,7 +252,7 @@ __host__ __device__ __forceinline__ uint32_t fold_slot(int table_b, int word) {
 }
 
 // Launchers (enqueue only).  Tables are bf16, nrows x vocab, column-major.
-// `hot` holds zeroed side buffers of hot.n x nrows floats each (hot.n may be 0); the update
+// `hot` holds zeroed side buffers of hot.n x side_stride(nrows) floats each (hot.n may be 0); the update
 // launchers leave them zeroed (they enqueue the narrowing kernel after the update kernel).
 hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
                            const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,

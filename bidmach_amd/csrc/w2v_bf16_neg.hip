@@ -43,8 +43,9 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       bscale[k] = 0.0f;
       if (k < nwb) {
         wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
-        load_col16<RP, ALIGNED, !EVAL>(b[k], B + (int64_t)wb[k] * d, lane, d);
-        if (!EVAL && wb[k] < hot.n) add_side_col<RP>(b[k], hot.sb + (int64_t)wb[k] * d, lane, d);
+        const bool fresh = !EVAL && wb[k] < hot.n;
+        load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d, fresh);
+        if (fresh) add_side_col<RP>(b[k], hot.sb + (int64_t)wb[k] * side_stride(d), lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
       } else {
 #pragma unroll
@@ -59,17 +60,18 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
     // every dot of the group
     float a[2 * RP], anext[2 * RP];
     int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa]);
-    load_col16<RP, ALIGNED, !EVAL>(a, A + (int64_t)wa * d, lane, d);
-    if (!EVAL && wa < hot.n) add_side_col<RP>(a, hot.sa + (int64_t)wa * d, lane, d);
+    load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d, !EVAL && wa < hot.n);
+    if (!EVAL && wa < hot.n) add_side_col<RP>(a, hot.sa + (int64_t)wa * side_stride(d), lane, d);
     for (int j = 0; j < nwa; ++j) {
       uint16_t* acol = A + (int64_t)wa * d;
       const bool ahot = !EVAL && wa < hot.n;
       int wanext = 0;
       if (j + 1 < nwa) {
         wanext = __builtin_amdgcn_readfirstlane(WA[i * nwa + j + 1]);
-        load_col16<RP, ALIGNED, !EVAL>(anext, A + (int64_t)wanext * d, lane, d);
+        load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d,
+                                !EVAL && wanext < hot.n);
         if (!EVAL && wanext < hot.n)
-          add_side_col<RP>(anext, hot.sa + (int64_t)wanext * d, lane, d);
+          add_side_col<RP>(anext, hot.sa + (int64_t)wanext * side_stride(d), lane, d);
       }
       float daa[2 * RP];
 #pragma unroll
@@ -98,7 +100,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       }
       if (!EVAL) {
         if (ahot)
-          atomic_add_side_col<RP>(hot.sa + (int64_t)wa * d, daa, lane, d);
+          atomic_add_side_col<RP>(hot.sa + (int64_t)wa * side_stride(d), daa, lane, d);
         else
           add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
                                  sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
@@ -117,7 +119,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         for (int k = 0; k < MAXB; ++k) {
           if (k < nwb) {
             if (wb[k] < hot.n)
-              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
+              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * side_stride(d), dbb[k], lane, d);
             else
               cas_first<RP>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
                             sr_key(seed, (uint32_t)i, (uint32_t)k), guess[k], found[k]);
@@ -134,7 +136,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         for (int k = 0; k < MAXB; ++k) {
           if (k < nwb) {
             if (wb[k] < hot.n)
-              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * d, dbb[k], lane, d);
+              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * side_stride(d), dbb[k], lane, d);
             else
               add_col16<RP, false>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
                                    sr_key(seed, (uint32_t)i, (uint32_t)k));

@@ -42,9 +42,9 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     const int ub = __builtin_amdgcn_readfirstlane(UB[i]);
     uint16_t* acol = A + (int64_t)w * d;
     float a[2 * RP], daa[2 * RP];
-    load_col16<RP, ALIGNED, !EVAL>(a, acol, lane, d);
     const bool ahot = !EVAL && w < hot.n;
-    if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)w * d, lane, d);
+    load_col16<RP, ALIGNED>(a, acol, lane, d, ahot);
+    if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)w * side_stride(d), lane, d);
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
@@ -64,8 +64,9 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       return hi + 1;
     };
     auto load_b = [&](float (&x)[2 * RP], int word) {
-      load_col16<RP, ALIGNED, !EVAL>(x, B + (int64_t)word * d, lane, d);
-      if (!EVAL && word < hot.n) add_side_col<RP>(x, hot.sb + (int64_t)word * d, lane, d);
+      const bool fresh = !EVAL && word < hot.n;
+      load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d, fresh);
+      if (fresh) add_side_col<RP>(x, hot.sb + (int64_t)word * side_stride(d), lane, d);
     };
     int wb = 0;
     int j = next_context(lo, wb);
@@ -97,7 +98,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
           db[r] = gb * a[r];
         }
         if (bhot)
-          atomic_add_side_col<RP>(hot.sb + (int64_t)wb * d, db, lane, d);
+          atomic_add_side_col<RP>(hot.sb + (int64_t)wb * side_stride(d), db, lane, d);
         else
           add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
@@ -109,7 +110,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     }
     if (!EVAL) {
       if (ahot)
-        atomic_add_side_col<RP>(hot.sa + (int64_t)w * d, daa, lane, d);
+        atomic_add_side_col<RP>(hot.sa + (int64_t)w * side_stride(d), daa, lane, d);
       else
         add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
     }
@@ -146,14 +147,16 @@ fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot) {
   const int w = blockIdx.x >> 1;
   const int table_b = blockIdx.x & 1;
   uint16_t* col = (table_b ? B : A) + (int64_t)w * d;
-  float* side = (table_b ? hot.sb : hot.sa) + (int64_t)w * d;
+  float* side = (table_b ? hot.sb : hot.sa) + (int64_t)w * side_stride(d);
   const uint32_t key = sr_key(seed, 0xFFFFFFFFU, fold_slot(table_b, w));
-  for (int e = threadIdx.x; e < d; e += kBlock) {
-    const float v = side[e];
+  for (int p = threadIdx.x; p < side_stride(d); p += kBlock) {
+    const int e = (p >> 7) * 128 + 2 * (p & 63) + ((p >> 6) & 1);   // the element stored at p
+    if (e >= d) continue;
+    const float v = side[p];
     if (v != 0.0f) {
       const float x = __builtin_bit_cast(float, (uint32_t)col[e] << 16) + v;
       col[e] = (uint16_t)sr_narrow(x, key, (uint32_t)e);
-      side[e] = 0.0f;
+      side[p] = 0.0f;
     }
   }
 }
