@@ -40,7 +40,7 @@ hipError_t side_buffers(int nrows, w2v::HotCols* out) {
   if (err != hipSuccess) return err;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   ThreadState& ts = t_state;
-  const size_t need = (size_t)2 * n * w2v::side_stride(nrows);
+  const size_t need = (size_t)2 * w2v::side_columns(n) * w2v::side_stride(nrows);
   if (ts.side16_floats[dev] < need) {
     if (ts.side16[dev] != nullptr) {
       err = hipStreamSynchronize(ts.stream);
@@ -63,7 +63,7 @@ hipError_t side_buffers(int nrows, w2v::HotCols* out) {
     ts.side16_floats[dev] = need;
   }
   out->sa = ts.side16[dev];
-  out->sb = ts.side16[dev] + (size_t)n * w2v::side_stride(nrows);
+  out->sb = ts.side16[dev] + (size_t)w2v::side_columns(n) * w2v::side_stride(nrows);
   return hipSuccess;
 }
 

@@ -204,7 +204,8 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
 // Frequent words.  Word ids are frequency ranks, so the first few hundred ids take most of the
 // updates of a call, and a compare-and-swap on a column that thousands of waves update at once
 // fails nearly every time.  The columns of the words below `n` therefore have an fp32 side
-// buffer each (sa for table A, sb for table B; n x side_stride(d) floats, zero between calls): while a call
+// buffer each (sa for table A, sb for table B; side_columns(n) x side_stride(d) floats, zero
+// between calls): while a call
 // runs, the value of such a column is widen(table) + side buffer, readers add the two in fp32,
 // and writers add their delta to the side buffer with float atomics, which need no retry.  A small
 // kernel at the end of the call narrows table + side buffer back into the table (one stochastic
@@ -245,6 +246,42 @@ __device__ __forceinline__ void atomic_add_side_col(float* side, const float (&d
   }
 }
 
+// The few most frequent words.  Requests to one cache line retire one after the other, and the
+// reads and float atomics of the most frequent word's side-buffer lines are the longest such
+// chain of a call.  The first kTopWords words therefore have kTopCopies side columns each (the
+// main one and kTopCopies - 1 more, stored after the hot.n main columns: copy c >= 1 of word w is
+// column hot.n + (c - 1) kTopWords + w): a writer adds to the copy its wave index selects, a
+// reader sums all copies, so the value read is still every update made so far while a line takes
+// a quarter of the atomics.  Used when hot.n >= kTopWords.
+constexpr int kTopWords = 8;
+constexpr int kTopCopies = 4;
+
+__host__ __device__ __forceinline__ int side_columns(int hot_n) {
+  return hot_n + (hot_n >= kTopWords ? (kTopCopies - 1) * kTopWords : 0);
+}
+
+template <int RP>
+__device__ __forceinline__ void read_side(float (&x)[2 * RP], const float* base, int hot_n, int w,
+                                          int lane, int d) {
+  const int64_t stride = side_stride(d);
+  add_side_col<RP>(x, base + (int64_t)w * stride, lane, d);
+  if (w < kTopWords && hot_n >= kTopWords) {
+#pragma unroll
+    for (int c = 1; c < kTopCopies; ++c)
+      add_side_col<RP>(x, base + ((int64_t)hot_n + (c - 1) * kTopWords + w) * stride, lane, d);
+  }
+}
+
+template <int RP>
+__device__ __forceinline__ void write_side(float* base, int hot_n, int w, int copy,
+                                           const float (&delta)[2 * RP], int lane, int d) {
+  const int64_t stride = side_stride(d);
+  int64_t column = w;
+  if (w < kTopWords && hot_n >= kTopWords && copy > 0)
+    column = (int64_t)hot_n + (copy - 1) * kTopWords + w;
+  atomic_add_side_col<RP>(base + column * stride, delta, lane, d);
+}
+
 // Slot of the end-of-call narrowing of a frequent word's column in the random-bit key (the unit
 // is 0xFFFFFFFF, which no token or group index reaches).
 __host__ __device__ __forceinline__ uint32_t fold_slot(int table_b, int word) {
@@ -252,7 +289,7 @@ __host__ __device__ __forceinline__ uint32_t fold_slot(int table_b, int word) {
 }
 
 // Launchers (enqueue only).  Tables are bf16, nrows x vocab, column-major.
-// `hot` holds zeroed side buffers of hot.n x side_stride(nrows) floats each (hot.n may be 0); the update
+// `hot` holds zeroed side buffers of side_columns(hot.n) x side_stride(nrows) floats each (hot.n may be 0); the update
 // launchers leave them zeroed (they enqueue the narrowing kernel after the update kernel).
 hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
                            const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,

@@ -29,6 +29,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
                 HotCols hot) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int copy = (blockIdx.x * kWavesPerBlock + wave) & (kTopCopies - 1);
   const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
   int64_t last = first + per_wave;
   if (last > n) last = n;
@@ -45,7 +46,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
         const bool fresh = !EVAL && wb[k] < hot.n;
         load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d, fresh);
-        if (fresh) add_side_col<RP>(b[k], hot.sb + (int64_t)wb[k] * side_stride(d), lane, d);
+        if (fresh) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
       } else {
 #pragma unroll
@@ -61,7 +62,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
     float a[2 * RP], anext[2 * RP];
     int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa]);
     load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d, !EVAL && wa < hot.n);
-    if (!EVAL && wa < hot.n) add_side_col<RP>(a, hot.sa + (int64_t)wa * side_stride(d), lane, d);
+    if (!EVAL && wa < hot.n) read_side<RP>(a, hot.sa, hot.n, wa, lane, d);
     for (int j = 0; j < nwa; ++j) {
       uint16_t* acol = A + (int64_t)wa * d;
       const bool ahot = !EVAL && wa < hot.n;
@@ -71,7 +72,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d,
                                 !EVAL && wanext < hot.n);
         if (!EVAL && wanext < hot.n)
-          add_side_col<RP>(anext, hot.sa + (int64_t)wanext * side_stride(d), lane, d);
+          read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
       }
       float daa[2 * RP];
 #pragma unroll
@@ -100,7 +101,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       }
       if (!EVAL) {
         if (ahot)
-          atomic_add_side_col<RP>(hot.sa + (int64_t)wa * side_stride(d), daa, lane, d);
+          write_side<RP>(hot.sa, hot.n, wa, copy, daa, lane, d);
         else
           add_col16<RP, ALIGNED>(acol, a, daa, lane, d,
                                  sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
@@ -119,7 +120,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         for (int k = 0; k < MAXB; ++k) {
           if (k < nwb) {
             if (wb[k] < hot.n)
-              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * side_stride(d), dbb[k], lane, d);
+              write_side<RP>(hot.sb, hot.n, wb[k], copy, dbb[k], lane, d);
             else
               cas_first<RP>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
                             sr_key(seed, (uint32_t)i, (uint32_t)k), guess[k], found[k]);
@@ -136,7 +137,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         for (int k = 0; k < MAXB; ++k) {
           if (k < nwb) {
             if (wb[k] < hot.n)
-              atomic_add_side_col<RP>(hot.sb + (int64_t)wb[k] * side_stride(d), dbb[k], lane, d);
+              write_side<RP>(hot.sb, hot.n, wb[k], copy, dbb[k], lane, d);
             else
               add_col16<RP, false>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d,
                                    sr_key(seed, (uint32_t)i, (uint32_t)k));

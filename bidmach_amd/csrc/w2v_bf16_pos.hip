@@ -31,6 +31,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
                 double* __restrict__ Retval, HotCols hot) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int copy = (blockIdx.x * kWavesPerBlock + wave) & (kTopCopies - 1);
   const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * per_wave;
   int64_t last = first + per_wave;
   if (last > n) last = n;
@@ -44,7 +45,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     float a[2 * RP], daa[2 * RP];
     const bool ahot = !EVAL && w < hot.n;
     load_col16<RP, ALIGNED>(a, acol, lane, d, ahot);
-    if (ahot) add_side_col<RP>(a, hot.sa + (int64_t)w * side_stride(d), lane, d);
+    if (ahot) read_side<RP>(a, hot.sa, hot.n, w, lane, d);
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
@@ -66,7 +67,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     auto load_b = [&](float (&x)[2 * RP], int word) {
       const bool fresh = !EVAL && word < hot.n;
       load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d, fresh);
-      if (fresh) add_side_col<RP>(x, hot.sb + (int64_t)word * side_stride(d), lane, d);
+      if (fresh) read_side<RP>(x, hot.sb, hot.n, word, lane, d);
     };
     int wb = 0;
     int j = next_context(lo, wb);
@@ -98,7 +99,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
           db[r] = gb * a[r];
         }
         if (bhot)
-          atomic_add_side_col<RP>(hot.sb + (int64_t)wb * side_stride(d), db, lane, d);
+          write_side<RP>(hot.sb, hot.n, wb, copy, db, lane, d);
         else
           add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
@@ -110,7 +111,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     }
     if (!EVAL) {
       if (ahot)
-        atomic_add_side_col<RP>(hot.sa + (int64_t)w * side_stride(d), daa, lane, d);
+        write_side<RP>(hot.sa, hot.n, w, copy, daa, lane, d);
       else
         add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
     }
@@ -147,16 +148,26 @@ fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot) {
   const int w = blockIdx.x >> 1;
   const int table_b = blockIdx.x & 1;
   uint16_t* col = (table_b ? B : A) + (int64_t)w * d;
-  float* side = (table_b ? hot.sb : hot.sa) + (int64_t)w * side_stride(d);
+  float* base = table_b ? hot.sb : hot.sa;
+  const int64_t stride = side_stride(d);
+  const int copies = (w < kTopWords && hot.n >= kTopWords) ? kTopCopies : 1;
   const uint32_t key = sr_key(seed, 0xFFFFFFFFU, fold_slot(table_b, w));
-  for (int p = threadIdx.x; p < side_stride(d); p += kBlock) {
+  for (int p = threadIdx.x; p < stride; p += kBlock) {
     const int e = (p >> 7) * 128 + 2 * (p & 63) + ((p >> 6) & 1);   // the element stored at p
     if (e >= d) continue;
-    const float v = side[p];
-    if (v != 0.0f) {
+    float v = base[(int64_t)w * stride + p];
+    bool any = v != 0.0f;
+    for (int c = 1; c < copies; ++c) {
+      const float u = base[((int64_t)hot.n + (c - 1) * kTopWords + w) * stride + p];
+      any = any || u != 0.0f;
+      v += u;
+    }
+    if (any) {
       const float x = __builtin_bit_cast(float, (uint32_t)col[e] << 16) + v;
       col[e] = (uint16_t)sr_narrow(x, key, (uint32_t)e);
-      side[p] = 0.0f;
+      base[(int64_t)w * stride + p] = 0.0f;
+      for (int c = 1; c < copies; ++c)
+        base[((int64_t)hot.n + (c - 1) * kTopWords + w) * stride + p] = 0.0f;
     }
   }
 }
