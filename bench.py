@@ -7,6 +7,11 @@ A step is one minibatch of the headline configuration (vocab 1M, dim 300, fp32, 
 Zipf(1.0) stream, window half-width 5, 5 negatives per positive drawn from unigram^0.75, groups of
 5 contexts) pushed through the two update operators.  Index arrays and tables are resident in HBM
 before the timed region starts.  Prints ONE JSON line.
+
+Other workloads (--workload) are the remaining configurations at their full shapes: dim 512 with
+window 10 and 15 negatives, the small vocab-10k configuration, forward-only scoring (--mode eval),
+and bfloat16 tables at vocab 3M (word2vecPosBf16 + word2vecNegBf16; its CPU baseline is the
+single-threaded bf16 oracle on a 300k-token sample).
 """
 import argparse
 import json
