@@ -256,9 +256,9 @@ def main():
         if evaluating:
             check(CUMACH.word2vecEvalPosAsync(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B,
                                               ret[0:1]), "word2vecEvalPos")
-        elif bf16:   # blocking call; the timer brackets the kernel on the launch stream
-            check(CUMACH.word2vecPosBf16(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B, lr,
-                                         args.vexp, 2 * s), "word2vecPosBf16")
+        elif bf16:
+            check(CUMACH.word2vecPosBf16Async(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], A, B,
+                                              lr, args.vexp, 2 * s), "word2vecPosBf16")
         elif MM:
             check(CUMACH.word2vecPosSlice(d, n, cfg["skip"], mb["W"], mb["LB"], mb["UB"], MM, lr,
                                           args.vexp, 0, args.slices, maxcols, args.head, False, 1),
@@ -273,9 +273,9 @@ def main():
             check(CUMACH.word2vecEvalNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                               mb["WB"], A, B, ret[1:2]), "word2vecEvalNeg")
         elif bf16:
-            check(CUMACH.word2vecNegBf16(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
-                                         mb["WB"], A, B, lr / cfg["nneg"], args.vexp, 2 * s + 1),
-                  "word2vecNegBf16")
+            check(CUMACH.word2vecNegBf16Async(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
+                                              mb["WB"], A, B, lr / cfg["nneg"], args.vexp,
+                                              2 * s + 1), "word2vecNegBf16")
         elif MM:
             check(CUMACH.word2vecNegSlice(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                           mb["WB"], MM, lr / cfg["nneg"], args.vexp, 0, args.slices,

@@ -401,9 +401,9 @@ int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* W
 
 // ---- bfloat16 tables ------------------------------------------------------------------------
 
-int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, unsigned short* A,
-                    unsigned short* B, float lrate, float vexp, unsigned long long seed) {
-  (void)shift;
+static int pos_bf16_impl(int nrows, int ncols, int* W, int* LB, int* UB, unsigned short* A,
+                         unsigned short* B, float lrate, float vexp, unsigned long long seed,
+                         bool sync) {
   if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
@@ -412,11 +412,25 @@ int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, u
   if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp,
                                      seed, hot),
-                true);
+                sync);
 }
 
-int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, unsigned short* A,
+int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, unsigned short* A,
                     unsigned short* B, float lrate, float vexp, unsigned long long seed) {
+  (void)shift;
+  return pos_bf16_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, true);
+}
+
+int word2vecPosBf16Async(int nrows, int ncols, int shift, int* W, int* LB, int* UB,
+                         unsigned short* A, unsigned short* B, float lrate, float vexp,
+                         unsigned long long seed) {
+  (void)shift;
+  return pos_bf16_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, false);
+}
+
+static int neg_bf16_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
+                         unsigned short* A, unsigned short* B, float lrate, float vexp,
+                         unsigned long long seed, bool sync) {
   if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb())
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
@@ -426,7 +440,18 @@ int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, un
   if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
                                      vexp, seed, hot),
-                true);
+                sync);
+}
+
+int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, unsigned short* A,
+                    unsigned short* B, float lrate, float vexp, unsigned long long seed) {
+  return neg_bf16_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, true);
+}
+
+int word2vecNegBf16Async(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
+                         unsigned short* A, unsigned short* B, float lrate, float vexp,
+                         unsigned long long seed) {
+  return neg_bf16_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, false);
 }
 
 int word2vecEvalPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB,

@@ -54,6 +54,8 @@ SYMBOLS = {
     "word2vecEvalNegAsync": (_I, _ENEG),
     "word2vecPosBf16": (_I, _POS + [ctypes.c_ulonglong]),
     "word2vecNegBf16": (_I, _NEG + [ctypes.c_ulonglong]),
+    "word2vecPosBf16Async": (_I, _POS + [ctypes.c_ulonglong]),
+    "word2vecNegBf16Async": (_I, _NEG + [ctypes.c_ulonglong]),
     "word2vecEvalPosBf16": (_I, _EPOS),
     "word2vecEvalNegBf16": (_I, _ENEG),
     "w2v_set_bf16_hot_words": (_I, [_I]),
@@ -262,6 +264,16 @@ class CUMACH:
     def word2vecNegBf16(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed):
         return load_library().word2vecNegBf16(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB), _ptr(A),
                                               _ptr(B), lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecPosBf16Async(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, seed):
+        return load_library().word2vecPosBf16Async(nrows, ncols, shift, _ptr(W), _ptr(LB),
+                                                   _ptr(UB), _ptr(A), _ptr(B), lrate, vexp, seed)
+
+    @staticmethod
+    def word2vecNegBf16Async(nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed):
+        return load_library().word2vecNegBf16Async(nrows, ncols, nwa, nwb, _ptr(WA), _ptr(WB),
+                                                   _ptr(A), _ptr(B), lrate, vexp, seed)
 
     @staticmethod
     def word2vecEvalPosBf16(nrows, ncols, shift, W, LB, UB, A, B, retVal):

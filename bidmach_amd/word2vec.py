@@ -256,8 +256,8 @@ class Word2Vec:
     def procPositives(self, nskip, words, lb, ub, model1, model2, lrate, vexp):
         nrows = model1.shape[1]
         if self.opts.storage == "bf16":
-            check(CUMACH.word2vecPosBf16(nrows, words.shape[0], nskip, words, lb, ub, model1,
-                                         model2, lrate, vexp, self._next_seed16()),
+            check(CUMACH.word2vecPosBf16Async(nrows, words.shape[0], nskip, words, lb, ub, model1,
+                                              model2, lrate, vexp, self._next_seed16()),
                   "word2vecPosBf16")
             return
         check(CUMACH.word2vecPosAsync(nrows, words.shape[0], nskip, words, lb, ub, model1, model2,
@@ -266,8 +266,9 @@ class Word2Vec:
     def procNegatives(self, nwa, nwb, wordsa, wordsb, modela, modelb, lrate, vexp):
         nrows = modela.shape[1]
         if self.opts.storage == "bf16":
-            check(CUMACH.word2vecNegBf16(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,
-                                         modela, modelb, lrate, vexp, self._next_seed16()),
+            check(CUMACH.word2vecNegBf16Async(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa,
+                                              wordsb, modela, modelb, lrate, vexp,
+                                              self._next_seed16()),
                   "word2vecNegBf16")
             return
         check(CUMACH.word2vecNegAsync(nrows, wordsa.shape[0] // nwa, nwa, nwb, wordsa, wordsb,

@@ -137,6 +137,13 @@ int word2vecPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB, u
                     unsigned short *B, float lrate, float vexp, unsigned long long seed);
 int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, unsigned short *A,
                     unsigned short *B, float lrate, float vexp, unsigned long long seed);
+/* Enqueue-only forms of the two update calls (completion: w2v_synchronize() or a timer). */
+int word2vecPosBf16Async(int nrows, int ncols, int shift, int *W, int *LB, int *UB,
+                         unsigned short *A, unsigned short *B, float lrate, float vexp,
+                         unsigned long long seed);
+int word2vecNegBf16Async(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB,
+                         unsigned short *A, unsigned short *B, float lrate, float vexp,
+                         unsigned long long seed);
 int word2vecEvalPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB,
                         unsigned short *A, unsigned short *B, double *Retval);
 int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB,

@@ -213,6 +213,51 @@ def test_unaligned_tables_take_the_halfword_path(gpu, oracle, hot):
     assert int(buf_a[0].item()) == 0 and int(buf_b[0].item()) == 0
 
 
+def test_column_offsets_beyond_2_to_31_elements_bf16(gpu, oracle):
+    """Tables of 7.3 M x 300 bfloat16: every column used starts beyond element 2^31 (byte 2^32).
+    With vexp = 0 neither the arithmetic nor the rounding keys depend on the id values, so the
+    oracle runs on a compact copy of the touched columns with the ids renumbered (and told that
+    none of them is a frequent word, as none of the large ids is)."""
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(92)
+    d, V, skip, nwa, nwb = 300, 7_300_000, 5, 5, 5
+    first = (1 << 31) // d + 1
+    n_ids = 4000
+    big = (first + rng.permutation(V - first)[:n_ids]).astype(np.int64)
+    assert (big * d > (1 << 31)).all()
+    Ac, Bc = tables16(rng, n_ids, d, 0.1)
+    A = torch.zeros((V, d), dtype=torch.int16, device="cuda")
+    B = torch.zeros((V, d), dtype=torch.int16, device="cuda")
+    idx = torch.from_numpy(big).cuda()
+    A[idx] = dev16(torch, Ac)
+    B[idx] = dev16(torch, Bc)
+    Wc, LB, UB = corpus.collision_free_pos(100, skip, 1100, np.random.default_rng(1))
+    WAc, WBc = corpus.collision_free_neg(200, nwa, nwb, 2000, np.random.default_rng(2))
+    WAc, WBc = WAc + 1100, WBc + 1100
+    Ao, Bo = Ac.copy(), Bc.copy()
+    oracle.word2vecPosBf16(d, Wc.shape[0], skip, Wc, LB, UB, Ao, Bo, 0.025, 0.0, 41, 0)
+    oracle.word2vecNegBf16(d, 200, nwa, nwb, WAc, WBc, Ao, Bo, 0.005, 0.0, 42, 0)
+    tobig = big.astype(np.int32)
+    assert CUMACH.word2vecPosBf16(d, Wc.shape[0], skip, dev(torch, tobig[Wc]), dev(torch, LB),
+                                  dev(torch, UB), A, B, 0.025, 0.0, 41) == 0
+    assert CUMACH.word2vecNegBf16(d, 200, nwa, nwb, dev(torch, tobig[WAc]),
+                                  dev(torch, tobig[WBc]), A, B, 0.005, 0.0, 42) == 0
+    assert_same_roundings(host16(A[idx]), Ao, Ac, "A")
+    assert_same_roundings(host16(B[idx]), Bo, Bc, "B")
+    assert (Ao != Ac).any() and (Bo != Bc).any()
+    ret = torch.zeros(1, dtype=torch.float64, device="cuda")
+    assert CUMACH.word2vecEvalPosBf16(d, Wc.shape[0], skip, dev(torch, tobig[Wc]),
+                                      dev(torch, LB), dev(torch, UB), A, B, ret) == 0
+    Ag, Bg = host16(A[idx]), host16(B[idx])
+    want = oracle.word2vecEvalPosBf16(d, Wc.shape[0], skip, Wc, LB, UB,
+                                      np.ascontiguousarray(Ag), np.ascontiguousarray(Bg))
+    assert float(ret.item()) == pytest.approx(want, rel=EVAL_RTOL)
+    # nothing else was touched
+    A[idx] = 0
+    B[idx] = 0
+    assert int(A.abs().max().item()) == 0 and int(B.abs().max().item()) == 0
+
+
 def test_table_conversions_match_torch(gpu):
     torch, _ = gpu
     from bidmach_amd.cumach import bf16_to_f32, f32_to_bf16
