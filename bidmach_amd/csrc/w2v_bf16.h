@@ -60,34 +60,29 @@ __device__ __forceinline__ uint32_t sr_narrow(float x, uint32_t key, uint32_t ro
   return (u + (sr_fmix32(key ^ (row * 0x9E3779B9U)) >> 16)) >> 16;
 }
 
-// A plain load may be served from the CU's own L1 or the XCD's own L2, which other CUs' and XCDs'
-// writes do not reach: a column that stays resident there is read as it was the first time.  The
-// columns of the frequent words do stay resident, so they (and their side buffers) are read with
-// device-scope loads (`fresh`); with plain loads and plain stores a frequent column ended as
-// whichever wave wrote last had left it.  Every other column is read with a plain load, like the
-// fp32 kernels': its line lives in an L2 for tens of microseconds at most, and the write-back does
-// not trust what was read -- the exchange compares against memory and repeats with the value
-// found.
-template <typename T>
-__device__ __forceinline__ T load_elt(const T* p, bool fresh) {
-  if (fresh) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return *p;
-}
-
+// Table columns are read with plain loads, like the fp32 kernels'.  A plain load may be served
+// from the CU's own L1 or the XCD's own L2, which other CUs' and XCDs' writes do not reach, so a
+// column that stays resident there is read as it was the first time.  That is harmless here for
+// two reasons.  The columns that do stay resident are the frequent words', and a frequent word's
+// table column does not change while a call runs: its updates go to its side buffer, which is
+// read with device-scope loads (add_side_col).  Every other column's line lives in an L2 for tens
+// of microseconds at most, and its write-back does not trust what was read: the exchange compares
+// against memory and repeats with the value found.  (With plain loads AND plain stores a frequent
+// column ended as whichever wave wrote last had left it.)
 template <int RP, bool ALIGNED>
 __device__ __forceinline__ void load_col16(float (&x)[2 * RP], const uint16_t* col, int lane,
-                                           int d, bool fresh) {
+                                           int d) {
 #pragma unroll
   for (int r = 0; r < RP; ++r) {
     const int e = r * 128 + 2 * lane;
     if (ALIGNED) {
       uint32_t v = 0;
-      if (e < d) v = load_elt(reinterpret_cast<const uint32_t*>(col + e), fresh);
+      if (e < d) v = *reinterpret_cast<const uint32_t*>(col + e);
       x[2 * r] = __builtin_bit_cast(float, v << 16);
       x[2 * r + 1] = __builtin_bit_cast(float, v & 0xFFFF0000U);
     } else {
-      const uint32_t lo = (e < d) ? load_elt(col + e, fresh) : 0U;
-      const uint32_t hi = (e + 1 < d) ? load_elt(col + e + 1, fresh) : 0U;
+      const uint32_t lo = (e < d) ? col[e] : 0U;
+      const uint32_t hi = (e + 1 < d) ? col[e + 1] : 0U;
       x[2 * r] = __builtin_bit_cast(float, lo << 16);
       x[2 * r + 1] = __builtin_bit_cast(float, hi << 16);
     }
@@ -187,7 +182,7 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
         const uintptr_t addr = reinterpret_cast<uintptr_t>(col + e);
         uint32_t* word = reinterpret_cast<uint32_t*>(addr & ~(uintptr_t)3);
         const int shift = (addr & 2) ? 16 : 0;
-        uint32_t guess = load_elt(word, true);
+        uint32_t guess = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         for (;;) {
           const float x = __builtin_bit_cast(float, ((guess >> shift) & 0xFFFFU) << 16) + delta[r];
           const uint32_t want = (guess & ~(0xFFFFU << shift)) |

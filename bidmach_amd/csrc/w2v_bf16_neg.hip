@@ -44,9 +44,8 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       bscale[k] = 0.0f;
       if (k < nwb) {
         wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
-        const bool fresh = !EVAL && wb[k] < hot.n;
-        load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d, fresh);
-        if (fresh) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
+        load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d);
+        if (!EVAL && wb[k] < hot.n) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
       } else {
 #pragma unroll
@@ -61,7 +60,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
     // every dot of the group
     float a[2 * RP], anext[2 * RP];
     int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa]);
-    load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d, !EVAL && wa < hot.n);
+    load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d);
     if (!EVAL && wa < hot.n) read_side<RP>(a, hot.sa, hot.n, wa, lane, d);
     for (int j = 0; j < nwa; ++j) {
       uint16_t* acol = A + (int64_t)wa * d;
@@ -69,8 +68,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
       int wanext = 0;
       if (j + 1 < nwa) {
         wanext = __builtin_amdgcn_readfirstlane(WA[i * nwa + j + 1]);
-        load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d,
-                                !EVAL && wanext < hot.n);
+        load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d);
         if (!EVAL && wanext < hot.n)
           read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
       }

@@ -44,7 +44,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     uint16_t* acol = A + (int64_t)w * d;
     float a[2 * RP], daa[2 * RP];
     const bool ahot = !EVAL && w < hot.n;
-    load_col16<RP, ALIGNED>(a, acol, lane, d, ahot);
+    load_col16<RP, ALIGNED>(a, acol, lane, d);
     if (ahot) read_side<RP>(a, hot.sa, hot.n, w, lane, d);
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
@@ -65,9 +65,8 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       return hi + 1;
     };
     auto load_b = [&](float (&x)[2 * RP], int word) {
-      const bool fresh = !EVAL && word < hot.n;
-      load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d, fresh);
-      if (fresh) read_side<RP>(x, hot.sb, hot.n, word, lane, d);
+      load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
+      if (!EVAL && word < hot.n) read_side<RP>(x, hot.sb, hot.n, word, lane, d);
     };
     int wb = 0;
     int j = next_context(lo, wb);
