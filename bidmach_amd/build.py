@@ -16,7 +16,11 @@ OBJ = os.path.join(CSRC, "_obj")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_NAME = "libbidmachhip-linux-x86_64.so"
 LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
-PROBE_PATH = os.path.join(LIB_DIR, "probe_atomics")
+# The name the reference's Java side asks its loader for (CUMACH.java:9 loads "bidmachcuda";
+# artefact libbidmachcuda-linux-x86_64.so, jni/src/Makefile:20-21): a link to the library, so a
+# BIDMach installation finds it under the name it already uses.
+ALIAS_NAME = "libbidmachcuda-linux-x86_64.so"
+ALIAS_PATH = os.path.join(LIB_DIR, ALIAS_NAME)
 
 SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
            "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_api.hip"]
@@ -59,24 +63,10 @@ def build(extra_flags=(), verbose=True, out=None):
     if verbose:
         print("built", out)
     if out == LIB_PATH:
-        build_probe(verbose)
+        if os.path.lexists(ALIAS_PATH):
+            os.remove(ALIAS_PATH)
+        os.symlink(LIB_NAME, ALIAS_PATH)
     return out
-
-
-def build_probe(verbose=True):
-    """The stand-alone device probe behind the atomic-scatter ceiling quoted in the design notes."""
-    cmd = [_hipcc(), "-O3", "-std=c++17", "--offload-arch=gfx950", "-munsafe-fp-atomics",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           os.path.join(CSRC, "probe_atomics.hip"), "-o", PROBE_PATH]
-    res = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
-    if err.strip():
-        sys.stderr.write(err + "\n")
-    if res.returncode != 0:
-        raise subprocess.CalledProcessError(res.returncode, cmd)
-    if verbose:
-        print("built", PROBE_PATH)
-    return PROBE_PATH
 
 
 if __name__ == "__main__":

@@ -40,10 +40,12 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
     int wb[MAXB];
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
-      wb[k] = 0;
+      // an id below zero (the positive stream's mark for a dropped word) skips its pairs, as in
+      // the fp32 kernels; wb[k] < 0 also stands for k >= nwb from here on
+      wb[k] = -1;
       bscale[k] = 0.0f;
-      if (k < nwb) {
-        wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
+      if (k < nwb) wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
+      if (wb[k] >= 0) {
         load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d);
         if (!EVAL && wb[k] < hot.n) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
@@ -60,25 +62,29 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
     // every dot of the group
     float a[2 * RP], anext[2 * RP];
     int wa = __builtin_amdgcn_readfirstlane(WA[i * nwa]);
-    load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d);
-    if (!EVAL && wa < hot.n) read_side<RP>(a, hot.sa, hot.n, wa, lane, d);
+    if (wa >= 0) {
+      load_col16<RP, ALIGNED>(a, A + (int64_t)wa * d, lane, d);
+      if (!EVAL && wa < hot.n) read_side<RP>(a, hot.sa, hot.n, wa, lane, d);
+    }
     for (int j = 0; j < nwa; ++j) {
       uint16_t* acol = A + (int64_t)wa * d;
       const bool ahot = !EVAL && wa < hot.n;
-      int wanext = 0;
+      int wanext = -1;
       if (j + 1 < nwa) {
         wanext = __builtin_amdgcn_readfirstlane(WA[i * nwa + j + 1]);
-        load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d);
-        if (!EVAL && wanext < hot.n)
-          read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
+        if (wanext >= 0) {
+          load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d);
+          if (!EVAL && wanext < hot.n)
+            read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
+        }
       }
       float daa[2 * RP];
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
-      const float ascale = EVAL ? 1.0f : scale_of(wa, vexp, smode);
+      const float ascale = (EVAL || wa < 0) ? 1.0f : scale_of(wa, vexp, smode);
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
-        if (k < nwb) {
+        if (wa >= 0 && wb[k] >= 0) {
           float part = 0.0f;
 #pragma unroll
           for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[k][r], part);
@@ -97,7 +103,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
           }
         }
       }
-      if (!EVAL) {
+      if (!EVAL && wa >= 0) {
         if (ahot)
           write_side<RP>(hot.sa, hot.n, wa, copy, daa, lane, d);
         else
@@ -116,7 +122,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         uint32_t guess[MAXB][RP], found[MAXB][RP];
 #pragma unroll
         for (int k = 0; k < MAXB; ++k) {
-          if (k < nwb) {
+          if (wb[k] >= 0) {
             if (wb[k] < hot.n)
               write_side<RP>(hot.sb, hot.n, wb[k], copy, dbb[k], lane, d);
             else
@@ -126,14 +132,14 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
         }
 #pragma unroll
         for (int k = 0; k < MAXB; ++k) {
-          if (k < nwb && wb[k] >= hot.n)
+          if (wb[k] >= 0 && wb[k] >= hot.n)
             cas_rest<RP>(B + (int64_t)wb[k] * d, dbb[k], lane, d,
                          sr_key(seed, (uint32_t)i, (uint32_t)k), guess[k], found[k]);
         }
       } else {
 #pragma unroll
         for (int k = 0; k < MAXB; ++k) {
-          if (k < nwb) {
+          if (wb[k] >= 0) {
             if (wb[k] < hot.n)
               write_side<RP>(hot.sb, hot.n, wb[k], copy, dbb[k], lane, d);
             else

@@ -183,11 +183,13 @@ void oracle_word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, const int *W
     for (k = 0; k < nwb; k++) {
       uint32_t key = oracle_bf16_key(seed, (uint32_t)i, (uint32_t)k);
       wb = WB[k + (int64_t)i * nwb];
+      if (wb < 0) continue; /* a dropped word skips its pairs, as in the fp32 library */
       ib = (int64_t)nrows * wb;
       bscale = pow(1 + wb, vexp);
       for (c = 0; c < nrows; c++) dbb[c] = 0;
       for (j = 0; j < nwa; j++) {
         wa = WA[j + (int64_t)i * nwa];
+        if (wa < 0) continue;
         ia = (int64_t)nrows * wa;
         ascale = pow(1 + wa, vexp);
         cv = 0;
@@ -212,6 +214,7 @@ void oracle_word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, const int *W
       uint32_t key = oracle_bf16_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j);
       ja = (int64_t)j * nrows;
       wa = WA[j + (int64_t)i * nwa];
+      if (wa < 0) continue;
       ia = (int64_t)nrows * wa;
       for (c = 0; c < nrows; c++) {
         if (wa < hot_n)
@@ -262,8 +265,10 @@ double oracle_word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, const 
   double dv = 0;
   for (ii = 0; ii < ncols; ii++) {
     for (k = 0; k < nwb; k++) {
+      if (WB[k + (int64_t)ii * nwb] < 0) continue;
       ib = (int64_t)nrows * WB[k + (int64_t)ii * nwb];
       for (j = 0; j < nwa; j++) {
+        if (WA[j + (int64_t)ii * nwa] < 0) continue;
         ia = (int64_t)nrows * WA[j + (int64_t)ii * nwa];
         cv = 0;
         for (c = 0; c < nrows; c++) cv += bf16_widen(A[c + ia]) * bf16_widen(B[c + ib]);

@@ -159,6 +159,36 @@ def test_neg_update_bf16(gpu, oracle, hot, vexp, d, nwa, nwb, G):
     assert (Ao != A).any() and (Bo != B).any()
 
 
+def test_neg_bf16_skips_pairs_with_a_dropped_word(gpu, oracle, hot):
+    """Ids below zero in WA / WB skip their pairs (update and forward sum): the touched columns
+    equal the oracle's, every other column keeps its bits."""
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(77)
+    d, V, G, nwa, nwb = 300, 20000, 300, 6, 5
+    A, B = tables16(rng, V, d, 0.5 / d ** 0.25)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    WA[rng.random(WA.shape[0]) < 0.2] = -1
+    WB[rng.random(WB.shape[0]) < 0.2] = -1
+    WA[:nwa] = -1
+    WB[nwb:2 * nwb] = -1
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.025, 0.5, 21, hot)
+    Ad, Bd = dev16(torch, A), dev16(torch, B)
+    assert CUMACH.word2vecNegBf16(d, G, nwa, nwb, dev(torch, WA), dev(torch, WB), Ad, Bd, 0.025,
+                                  0.5, 21) == 0
+    assert_same_roundings(host16(Ad), Ao, A, "A")
+    assert_same_roundings(host16(Bd), Bo, B, "B")
+    keep_a = (Ao == A).all(axis=1)
+    keep_b = (Bo == B).all(axis=1)
+    assert keep_a.sum() > V - G * nwa and keep_b.sum() > V - G * nwb
+    assert (host16(Ad)[keep_a] == A[keep_a]).all() and (host16(Bd)[keep_b] == B[keep_b]).all()
+    want = oracle.word2vecEvalNegBf16(d, G, nwa, nwb, WA, WB, A, B)
+    ret = torch.zeros(1, dtype=torch.float64, device="cuda")
+    assert CUMACH.word2vecEvalNegBf16(d, G, nwa, nwb, dev(torch, WA), dev(torch, WB),
+                                      dev16(torch, A), dev16(torch, B), ret) == 0
+    assert float(ret.item()) == pytest.approx(want, rel=EVAL_RTOL)
+
+
 def test_updates_within_1e_4_of_the_fp32_oracle_at_initial_scale(gpu, oracle):
     # tables as the reference starts them (Word2Vec.scala:112-117) plus a first update's worth
     # in the zero table; below 2**-6 one bfloat16 step is at most 6.1e-5, i.e. under 1e-4

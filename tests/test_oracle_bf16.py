@@ -134,6 +134,46 @@ def test_neg_update_is_a_rounding_of_the_fp32_oracle(oracle, vexp, d, nwa, nwb, 
     assert (A16 != A).any() and (B16 != B).any()
 
 
+@pytest.mark.parametrize("hot", [0, 1500])
+def test_neg_skips_pairs_with_a_dropped_word(oracle, hot):
+    # ids below zero (the positive stream's mark for a dropped word) skip every pair they take
+    # part in: pinned against the fp32 oracle's filtered negative pass, which drops them too
+    rng = np.random.default_rng(77)
+    d, V, G, nwa, nwb = 40, 4000, 80, 6, 5
+    A, B = tables16(rng, V, d, 0.5 / d ** 0.25)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    WA[rng.random(WA.shape[0]) < 0.2] = -1
+    WB[rng.random(WB.shape[0]) < 0.2] = -1
+    WA[:nwa] = -1                      # a group without A words
+    WB[nwb:2 * nwb] = -1               # a group without B words
+    A32, B32 = cpumach.bf16_widen(A).copy(), cpumach.bf16_widen(B).copy()
+    oracle.word2vecNegFilt(d, G, V, nwa, nwb, WA, WB, A32, B32, 0.025, 0.5, 1)
+    A16, B16 = A.copy(), B.copy()
+    oracle.word2vecNegBf16(d, G, nwa, nwb, WA, WB, A16, B16, 0.025, 0.5, 5, hot)
+    assert neighbours_ok(A16, A32) and neighbours_ok(B16, B32)
+    assert (A16 != A).any() and (B16 != B).any()
+    # columns of words whose every partner was dropped, and unused columns, keep their bits
+    same_a = (A32 == cpumach.bf16_widen(A)).all(axis=1)
+    same_b = (B32 == cpumach.bf16_widen(B)).all(axis=1)
+    assert (A16[same_a] == A[same_a]).all() and (B16[same_b] == B[same_b]).all()
+    want = oracle.word2vecEvalNeg(d, G, nwa, nwb, np.where(WA < 0, 0, WA).astype(np.int32),
+                                  np.where(WB < 0, 0, WB).astype(np.int32),
+                                  cpumach.bf16_widen(A), cpumach.bf16_widen(B), 1)
+    got = oracle.word2vecEvalNegBf16(d, G, nwa, nwb, WA, WB, A, B)
+    assert got > want                  # fewer (negative) terms than with the ids patched to 0
+    # forward sum over the kept pairs only: brute force
+    a32, b32 = cpumach.bf16_widen(A).astype(np.float64), cpumach.bf16_widen(B).astype(np.float64)
+    tot = 0.0
+    for i in range(G):
+        for k in range(nwb):
+            for j in range(nwa):
+                wa, wb = WA[i * nwa + j], WB[i * nwb + k]
+                if wa >= 0 and wb >= 0:
+                    s = float(a32[wa] @ b32[wb])
+                    tot += np.log(max(1.0 - 1.0 / (1.0 + np.exp(-s)), 1e-40))
+    assert got == pytest.approx(tot, rel=1e-6)
+
+
 def test_mean_over_seeds_approaches_the_fp32_result(oracle):
     # the expectation of the stored value is the fp32 value: averaged over many seeds the bf16
     # result comes far closer to the fp32 oracle than one bf16 step
