@@ -2,7 +2,7 @@
 (src/main/scala/BIDMach/networks/Word2Vec.scala:1332-1394 of the reference).
 
 Layout: a header line "<nwords> <dim>\\n", then per word its string, one space, `dim` values and a
-newline.  Text files print each value with "%g " (:1385); binary files hold raw IEEE floats.  The
+newline.  Text files print each value with Java's "%g " (:1385; java_g below); binary files hold raw IEEE floats.  The
 reference writes binary values through java.io.DataOutputStream.writeFloat (:1383) and reads them
 with DataInputStream.readFloat (:1350), i.e. BIG-endian, whereas Google's own tool writes
 little-endian; `byteorder` selects which (default: the reference's).
@@ -10,7 +10,47 @@ little-endian; `byteorder` selects which (default: the reference's).
 A model matrix here is the (vocab, dim) C-order array the operators use (word w's vector is row
 w), which is the reference's dim x vocab column-major FMat.
 """
+import math
+from decimal import Decimal
+
 import numpy as np
+
+
+def java_g(v):
+    """One value as the reference's writer prints it: Scala's `"%g " format x`
+    (Word2Vec.scala:1385) is java.util.Formatter's general-scientific conversion with the default
+    precision 6, applied to the float widened to double.  Its rules: round to 6 significant
+    digits, half up on the decimal digits; if the rounded magnitude is in [1e-4, 1e6) print it as
+    a plain decimal with 6 significant digits in all, trailing zeros kept and no decimal point
+    when no fraction digit is left ("0.100000", "12.3457", "123457"); otherwise as d.ddddde+xx
+    with a sign and at least two exponent digits ("1.00000e-05", "1.23457e+08").  Zero prints as
+    "0.00000", not-a-number as "NaN", the infinities as "Infinity" / "-Infinity".  Unlike C's and
+    Python's %g nothing is stripped."""
+    x = float(v)
+    if math.isnan(x):
+        return "NaN"
+    if math.isinf(x):
+        return "Infinity" if x > 0 else "-Infinity"
+    sign = "-" if math.copysign(1.0, x) < 0 else ""
+    x = abs(x)
+    if x == 0.0:
+        return sign + "0.00000"
+    # the shortest decimal digits that identify the double, which is what Java rounds
+    t = Decimal(repr(x)).as_tuple()
+    all_digits = "".join(map(str, t.digits)).lstrip("0")
+    exp10 = len(t.digits) + t.exponent - 1 - (len(t.digits) - len(all_digits))
+    digits = (all_digits + "000000")[:6]
+    if len(all_digits) > 6 and all_digits[6] >= "5":      # half up
+        n = int(digits) + 1
+        if n == 1000000:
+            n, exp10 = 100000, exp10 + 1
+        digits = "%06d" % n
+    if -4 <= exp10 < 6:
+        if exp10 >= 0:
+            whole, frac = digits[:exp10 + 1], digits[exp10 + 1:]
+            return sign + whole + ("." + frac if frac else "")
+        return sign + "0." + "0" * (-exp10 - 1) + digits
+    return "%s%s.%se%s%02d" % (sign, digits[0], digits[1:], "-" if exp10 < 0 else "+", abs(exp10))
 
 
 def saveGoogleW2V(words, mod, fname, binary=False, byteorder=">"):
@@ -25,7 +65,7 @@ def saveGoogleW2V(words, mod, fname, binary=False, byteorder=">"):
             if binary:
                 f.write(mod[i].astype(byteorder + "f4").tobytes())
             else:
-                f.write("".join("%g " % v for v in mod[i]).encode())
+                f.write("".join(java_g(v) + " " for v in mod[i]).encode())
             f.write(b"\n")
 
 
