@@ -66,6 +66,8 @@ def build(extra_flags=(), verbose=True, out=None):
         if os.path.lexists(ALIAS_PATH):
             os.remove(ALIAS_PATH)
         os.symlink(LIB_NAME, ALIAS_PATH)
+        # where a JDK is installed the JNI glue takes the alias's place (jni/Makefile)
+        subprocess.check_call(["make", "-s", "-C", os.path.join(os.path.dirname(HERE), "jni")])
     return out
 
 

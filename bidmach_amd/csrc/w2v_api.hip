@@ -505,6 +505,30 @@ int w2v_set_stream(void* stream) {
 void* w2v_get_stream(void) { return reinterpret_cast<void*>(t_state.stream); }
 int w2v_synchronize(void) { return (int)hipStreamSynchronize(t_state.stream); }
 
+int w2v_release_thread(void) {
+  ThreadState& ts = t_state;
+  bool held = false;
+  for (int dev = 0; dev < kMaxDevices; ++dev)
+    held = held || ts.partials[dev] || ts.shadow[dev] || ts.side16[dev];
+  if (!held) return 0;
+  hipError_t first = hipStreamSynchronize(ts.stream);   // nothing may still be using the scratch
+  auto release = [&first](auto*& p) {
+    if (p != nullptr) {
+      const hipError_t err = hipFree(p);
+      if (first == hipSuccess) first = err;
+      p = nullptr;
+    }
+  };
+  for (int dev = 0; dev < kMaxDevices; ++dev) {
+    release(ts.partials[dev]);
+    ts.capacity[dev] = 0;
+    release(ts.shadow[dev]);
+    release(ts.side16[dev]);
+    ts.side16_floats[dev] = 0;
+  }
+  return (int)first;
+}
+
 int w2v_set_max_workgroups(int n) {
   w2v::set_max_workgroups(n);
   return 0;

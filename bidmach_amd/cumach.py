@@ -67,6 +67,7 @@ SYMBOLS = {
     "w2v_set_stream": (_I, [_P]),
     "w2v_get_stream": (_P, []),
     "w2v_synchronize": (_I, []),
+    "w2v_release_thread": (_I, []),
     "w2v_set_max_workgroups": (_I, [_I]),
     "w2v_get_max_workgroups": (_I, []),
     "w2v_set_hot_update_mode": (_I, [_I]),

@@ -173,6 +173,14 @@ int w2v_set_stream(void *stream);
 void *w2v_get_stream(void);
 int w2v_synchronize(void);
 
+/* Frees the device scratch memory the calling thread holds (per device: the forward sums'
+ * partial buffer, the shadow and occurrence-count buffers of the update operators, the fp32 side
+ * buffers of the bfloat16 operators; allocated on the thread's first calls) after waiting for the
+ * thread's launch stream.  The next call allocates it again.  Call it before a worker thread that
+ * used the library ends (a JVM thread pool, say): thread-local scratch is not freed by thread
+ * exit.  No counterpart in the reference, whose launchers keep no state. */
+int w2v_release_thread(void);
+
 /* Upper bound on the workgroups of the two update kernels, process-wide (0 = as many as the
  * device holds, the default).  The update kernels are persistent: each workgroup walks a
  * contiguous range of the minibatch in order, so this bounds the number of work units in flight

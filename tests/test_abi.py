@@ -60,3 +60,21 @@ def test_limits_and_floor_without_gpu():
 def test_missing_library_fails_loudly(tmp_path):
     with pytest.raises(cumach.W2VLibraryError):
         cumach.load_library(str(tmp_path / "nope.so"))
+
+
+def test_jni_glue_binds_the_reference_natives_to_declared_functions():
+    """jni/cumach_w2v_jni.cpp (built only where a JDK is installed) defines one
+    Java_edu_berkeley_bid_CUMACH_<name> per native the reference's Java class declares for this
+    path (CUMACH.java:90,92,94,96,98) and forwards each to the C function of the same name."""
+    text = open(os.path.join(ROOT, "jni", "cumach_w2v_jni.cpp")).read()
+    declared = declared_functions()
+    for n in ("word2vecPos", "word2vecNeg", "word2vecNegFilt", "word2vecEvalPos",
+              "word2vecEvalNeg"):
+        assert re.search(r"Java_edu_berkeley_bid_CUMACH_%s\(" % n, text), n
+        assert re.search(r"return %s\(" % n, text), n
+        assert n in declared
+    assert "JNI_OnLoad" in text and "nativePointer" in text and "byteOffset" in text
+
+
+def test_release_thread_without_scratch_is_a_no_op():
+    assert cumach.load_library().w2v_release_thread() == 0

@@ -163,3 +163,53 @@ def test_max_workgroups_knob_does_not_change_results(lib, oracle):
             assert np.abs(Bd.cpu().numpy() - Bo).max() <= 1e-4
     finally:
         lib.w2v_set_max_workgroups(0)
+
+
+def test_release_thread_frees_the_scratch_and_later_calls_still_work(lib, oracle):
+    """A worker thread calls the operators (which allocates its scratch), releases it, and the
+    device's free memory is back where it was; calls after a release allocate again and give the
+    oracle's result."""
+    import torch
+    rng = np.random.default_rng(8)
+    d, V, G, nwa, nwb = 300, 9000, 200, 5, 5
+    A = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.1).astype(np.float32)
+    WA, WB = corpus.collision_free_neg(G, nwa, nwb, V, rng)
+    A16 = torch.zeros((V, d), dtype=torch.int16, device="cuda")
+    B16 = torch.zeros((V, d), dtype=torch.int16, device="cuda")
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    WAd, WBd = torch.from_numpy(WA).cuda(), torch.from_numpy(WB).cuda()
+    ret = torch.zeros(1, dtype=torch.float64, device="cuda")
+    result = {}
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    def worker():
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        ok = lib.word2vecNeg(d, G, nwa, nwb, ptr(WAd), ptr(WBd), ptr(Ad), ptr(Bd), 0.005, 0.5) == 0
+        ok &= lib.word2vecEvalNegF64(d, G, nwa, nwb, ptr(WAd), ptr(WBd), ptr(Ad), ptr(Bd),
+                                     ptr(ret)) == 0
+        ok &= lib.word2vecNegBf16(d, G, nwa, nwb, ptr(WAd), ptr(WBd), ptr(A16), ptr(B16), 0.005,
+                                  0.5, 3) == 0
+        held = free0 - torch.cuda.mem_get_info()[0]
+        ok &= lib.w2v_release_thread() == 0
+        after = free0 - torch.cuda.mem_get_info()[0]
+        ok &= lib.w2v_release_thread() == 0          # a second release has nothing to free
+        # and the thread can go on: scratch is allocated again
+        ok &= lib.word2vecNeg(d, G, nwa, nwb, ptr(WAd), ptr(WBd), ptr(Ad), ptr(Bd), 0.005, 0.5) == 0
+        ok &= lib.w2v_release_thread() == 0
+        result.update(ok=bool(ok), held=held, after=after)
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert result["ok"]
+    assert result["held"] >= 8 << 20, result       # the thread's scratch was real device memory
+    assert result["after"] <= 2 << 20, result      # and the release gave it back
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.005, 0.5, 1)
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.005, 0.5, 1)
+    assert np.abs(Ad.cpu().numpy() - Ao).max() <= 1e-4
+    assert np.abs(Bd.cpu().numpy() - Bo).max() <= 1e-4
