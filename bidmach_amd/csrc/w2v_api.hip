@@ -27,6 +27,7 @@ thread_local ThreadState t_state;
 std::atomic<double> g_eval_floor{1.0e-40};
 std::atomic<int> g_bf16_hot_words{1024};
 constexpr int kMaxBf16HotWords = 4096;
+constexpr int kMaxNwbBf16 = 8;   // the bfloat16 negative kernels hold every B column in registers
 
 // Per-thread, per-device fp32 side buffers for the frequent words of bf16 tables (A's then B's),
 // zeroed when allocated; the update launchers leave them zeroed.  They only grow.
@@ -431,7 +432,7 @@ int word2vecPosBf16Async(int nrows, int ncols, int shift, int* W, int* LB, int* 
 static int neg_bf16_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
                          unsigned short* A, unsigned short* B, float lrate, float vexp,
                          unsigned long long seed, bool sync) {
-  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb())
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > kMaxNwbBf16)
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
@@ -467,7 +468,7 @@ int word2vecEvalPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* U
 
 int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
                         unsigned short* A, unsigned short* B, double* Retval) {
-  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || !Retval)
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > kMaxNwbBf16 || !Retval)
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;

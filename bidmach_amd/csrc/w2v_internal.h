@@ -94,6 +94,15 @@ hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int
                       const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
                       Shadow shadow);
 
+// The same pass for groups with more than 8 B words (w2v_neg_wide.hip): the group's A columns are
+// staged in LDS, so nwa * ceil(nrows / 64) is bounded (hipErrorInvalidValue beyond, about 300).
+hipError_t launch_neg_wide(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                           const int* WA, const int* WB, float* A, float* B, float lrate,
+                           float vexp);
+hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                 const int* WA, const int* WB, const SliceMap& m, float lrate,
+                                 float vexp);
+
 // Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
 // and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or
 // Retval64[0] (double, added into).  Either output pointer may be null.

@@ -56,22 +56,24 @@ neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
     if (lane < nwa) wal0 = WA[unit * nwa + lane];
   }
   for (; unit < g_end; unit += kWavesPerBlock) {
-    float b[MAXB][R];
-    int wb[MAXB];
-#pragma unroll
-    for (int k = 0; k < MAXB; ++k) {
-      wb[k] = -1;
-      if (k < nwb) {
-        wb[k] = read_lane(wbl, k);
-        if (wb[k] >= 0) load_col<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
-      }
-    }
     // ids of this wave's next group, in flight while this group is scored
     const int64_t next = unit + kWavesPerBlock;
     int wbl_next = -1, wal_next = -1;
     if (next < g_end) {
       if (lane < nwb) wbl_next = WB[next * nwb + lane];
       if (lane < nwa) wal_next = WA[next * nwa + lane];
+    }
+    // MAXB columns of B at a time (one trip unless nwb > MAXB)
+    for (int kb = 0; kb < nwb; kb += MAXB) {
+    float b[MAXB][R];
+    int wb[MAXB];
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      wb[k] = -1;
+      if (kb + k < nwb) {
+        wb[k] = read_lane(wbl, kb + k);
+        if (wb[k] >= 0) load_col<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
+      }
     }
     for (int jbase = 0; jbase < nwa; jbase += kWave) {
       int wal = wal0;
@@ -110,6 +112,7 @@ neg_eval_kernel(int d, int ngroups, int nwa, int nwb, int64_t groups_per_wg,
         }
         if (live) lsum += log(fmax(1.0 - (double)sat_sigmoid(pre), floorv));
       }
+    }
     }
     wbl = wbl_next;
     wal0 = wal_next;
@@ -154,23 +157,33 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
     const float sbl = wbl >= 0 ? scale_of(wbl, vexp, smode) : 0.0f;
     // a word that occurs twice in the group would have two plain updates in flight: not rare
     bool lone_b = true;
+    if (nwb <= MAXB) {
 #pragma unroll
-    for (int k = 0; k < MAXB; ++k)
-      if (k < nwb && k != lane && read_lane(wbl, k) == wbl) lone_b = false;
+      for (int k = 0; k < MAXB; ++k)
+        if (k < nwb && k != lane && read_lane(wbl, k) == wbl) lone_b = false;
+    } else {
+      for (int k = 0; k < nwb; ++k)
+        if (k != lane && read_lane(wbl, k) == wbl) lone_b = false;
+    }
     const uint64_t rare_b = __ballot(wbl >= 0 && lone_b && is_rare(shadow, wbl));
     // tickets for the writes to hot B columns at the end of the group, taken now
     const unsigned tkb = hot_ticket(shadow, 0, slot, (wbl >= 0 && wbl < kHotWords) ? wbl : -1);
 
+    // MAXB columns of B at a time.  The launcher sends groups with nwb > MAXB to the kernel of
+    // w2v_neg_wide.hip, so this loop makes one trip: with more, the A columns would be read again
+    // on every trip with the group's own earlier deltas in them, which the reference's order
+    // (A written after the group's last dot, BIDMach_CPUMACH.c:248-254) does not allow.
+    for (int kb = 0; kb < nwb; kb += MAXB) {
     float b[MAXB][R];
     float dbb[MAXB][R];
     int wb[MAXB];
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       wb[k] = -1;
-      if (k < nwb) {
-        wb[k] = read_lane(wbl, k);
+      if (kb + k < nwb) {
+        wb[k] = read_lane(wbl, kb + k);
         if (wb[k] >= 0) {
-          if ((rare_b >> k) & 1)
+          if ((rare_b >> (kb + k)) & 1)
             load_col_fresh<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
           else
             load_col_ref<R>(b[k], table_ref(B, wb[k], d), shadow, 0, lane, d);
@@ -190,7 +203,10 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
         for (int j = 0; j < jend; ++j)
           if (j != lane && read_lane(wal, j) == wal) lone_a = false;
       }
-      const uint64_t rare_a = __ballot(wal >= 0 && lone_a && is_rare(shadow, wal));
+      // (an A word updated on several trips is not rare: its plain updates would be in flight
+      // together)
+      const uint64_t rare_a =
+          __ballot(wal >= 0 && lone_a && nwb <= MAXB && is_rare(shadow, wal));
       const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -233,7 +249,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
             for (int k = 0; k < MAXB; ++k) {
               if (wb[k] >= 0) {
                 const float g = read_lane(gl, c * MAXB + k);
-                const float bs = read_lane(sbl, k);
+                const float bs = read_lane(sbl, kb + k);
                 axpy<R>(dbb[k], bs * g, a[c]);
                 axpy<R>(daa, as * g, b[k]);
               }
@@ -251,12 +267,13 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       if (wb[k] >= 0) {
-        if ((rare_b >> k) & 1)
+        if ((rare_b >> (kb + k)) & 1)
           store_sum_col<R>(B + (int64_t)wb[k] * d, b[k], dbb[k], lane, d);
         else
           scatter_add_ref<R>(table_ref(B, wb[k], d), shadow, 0, slot, dbb[k], lane, d,
-                             read_lane(tkb, k));
+                             read_lane(tkb, kb + k));
       }
+    }
     }
   }
 }
@@ -367,7 +384,8 @@ hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, 
   return hipGetLastError();
 }
 
-constexpr int kMaxNwb = 8;
+constexpr int kMaxTileB = 8;     // B columns a wave holds in registers at once
+constexpr int kMaxNwb = kWave;   // lane k of a wave holds the group's k-th B word
 int max_nwb() { return kMaxNwb; }
 
 // A columns gathered per chunk, sized so that b, dbb and the chunk stay near 100 registers.
@@ -437,7 +455,7 @@ static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int idlim
                                               partials, nparts)
   if (nwb <= 2) W2V_NEG_DISPATCH(2);
   if (nwb <= 5) W2V_NEG_DISPATCH(5);
-  if (nwb <= kMaxNwb) W2V_NEG_DISPATCH(kMaxNwb);
+  if (nwb <= kMaxNwb) W2V_NEG_DISPATCH(kMaxTileB);
 #undef W2V_NEG_DISPATCH
   return hipErrorInvalidValue;
 }
@@ -445,6 +463,8 @@ static hipError_t launch_neg_r(hipStream_t stream, int d, int ngroups, int idlim
 hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                       const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
                       Shadow shadow) {
+  if (nwb > kMaxTileB)
+    return launch_neg_wide(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp);
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
 #define CALL(R)                                                                                   \

@@ -158,15 +158,18 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     uint64_t rare_b = 0;
     if (TRAIN && shadow.rare_max > 0) {
       bool lone = true;
-#pragma unroll
-      for (int k = 0; k < MAXB; ++k)
-        if (k < nwb && k != lane && read_lane(wbl, k) == wbl) lone = false;
+      for (int k = 0; k < nwb; ++k)
+        if (k != lane && read_lane(wbl, k) == wbl) lone = false;
       rare_b = __ballot(lone && pbl.hot < 0 && tables.written(pbl.flags) && is_rare(shadow, wbl));
     }
     // tickets for the writes to hot B columns at the end of the group, taken now
     const unsigned tkb =
         (TRAIN && tables.written(pbl.flags)) ? hot_ticket(shadow, 0, slot, pbl.hot) : 0u;
 
+    // MAXB columns of B at a time: several trips only in the forward-only instance (training
+    // groups with nwb > MAXB go to the kernel of w2v_neg_wide.hip, which keeps the reference's
+    // rule that every dot of a group sees the A columns as they were when the group started)
+    for (int kb = 0; kb < nwb; kb += MAXB) {
     float b[MAXB][R];
     float dbb[MAXB][R];
     ColRef rb[MAXB];
@@ -175,11 +178,11 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     for (int k = 0; k < MAXB; ++k) {
       fb[k] = 0;
       rb[k] = ColRef{nullptr, -1, 0};
-      if (k < nwb) {
-        rb[k] = read_lane_ref(pbl, k);
+      if (kb + k < nwb) {
+        rb[k] = read_lane_ref(pbl, kb + k);
         fb[k] = rb[k].flags;
         if (fb[k] != 0) {
-          if ((rare_b >> k) & 1)
+          if ((rare_b >> (kb + k)) & 1)
             load_col_fresh<R>(b[k], rb[k].col, lane, d);
           else
             load_col_ref<R>(b[k], rb[k], shadow, 0, lane, d);
@@ -201,7 +204,8 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
         bool lone = true;
         for (int j = 0; j < jend; ++j)
           if (j != lane && read_lane(wal, j) == wal) lone = false;
-        rare_a = __ballot(lone && pal.hot < 0 && tables.written(pal.flags) && is_rare(shadow, wal));
+        rare_a = __ballot(lone && nwb <= MAXB && pal.hot < 0 && tables.written(pal.flags) &&
+                          is_rare(shadow, wal));
       }
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -251,7 +255,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
               for (int k = 0; k < MAXB; ++k) {
                 if (fb[k] != 0 && tables.trained(fa[c], fb[k])) {
                   const float g = read_lane(gl, c * MAXB + k);
-                  const float bs = read_lane(sbl, k);
+                  const float bs = read_lane(sbl, kb + k);
                   axpy<R>(dbb[k], bs * g, a[c]);
                   axpy<R>(daa, as * g, b[k]);
                 }
@@ -271,11 +275,12 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
     if (TRAIN) {
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
-        if ((rare_b >> k) & 1)
+        if (kb + k < nwb && ((rare_b >> (kb + k)) & 1))
           store_sum_col<R>(rb[k].col, b[k], dbb[k], lane, d);
         else if (fb[k] != 0 && tables.written(fb[k]))
-          scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d, read_lane(tkb, k));
+          scatter_add_ref<R>(rb[k], shadow, 0, slot, dbb[k], lane, d, read_lane(tkb, kb + k));
       }
+    }
     }
   }
 
@@ -361,7 +366,7 @@ static hipError_t launch_slice_neg_r(hipStream_t stream, int d, int ngroups, int
   if (nwb <= 5)
     return launch_slice_neg_rb<R, 5, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
                                             floorv, partials, nparts, shadow);
-  if (nwb <= 8)
+  if (nwb <= max_nwb())
     return launch_slice_neg_rb<R, 8, TRAIN>(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
                                             floorv, partials, nparts, shadow);
   return hipErrorInvalidValue;
@@ -389,6 +394,8 @@ hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, int shift,
 hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                             const int* WA, const int* WB, const SliceMap& m, float lrate,
                             float vexp, Shadow shadow) {
+  if (nwb > 8)
+    return launch_slice_neg_wide(stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate, vexp);
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
   hipError_t err = hipSuccess;

@@ -132,7 +132,7 @@ int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int *WA, int *W
  * in flight).  With an odd nrows or a table on an odd 2-byte boundary the word that holds the
  * first or last element of a table reaches 2 bytes outside it; those bytes are written back
  * unchanged and must be addressable (they are inside any allocation the table is a view of).
- * nwb <= w2v_max_nwb(). */
+ * nwb <= 8. */
 int word2vecPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB, unsigned short *A,
                     unsigned short *B, float lrate, float vexp, unsigned long long seed);
 int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, unsigned short *A,
@@ -223,7 +223,8 @@ int w2v_get_hot_update_mode(void);
 int w2v_set_rare_update_mode(int mode);
 int w2v_get_rare_update_mode(void);
 
-/* Limits of the kernels: largest nrows and largest nwb. */
+/* Limits of the kernels: largest nrows and largest nwb (fp32 tables; the bfloat16 operators take
+ * nwb <= 8). */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
 

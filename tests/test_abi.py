@@ -50,7 +50,7 @@ def test_header_compiles_as_c():
 def test_limits_and_floor_without_gpu():
     lib = cumach.load_library()
     assert lib.w2v_max_rows() == 1280
-    assert lib.w2v_max_nwb() == 8
+    assert lib.w2v_max_nwb() == 64
     assert lib.w2v_get_eval_floor() == 1.0e-40
     lib.w2v_set_eval_floor(1.0e-20)
     assert lib.w2v_get_eval_floor() == 1.0e-20

@@ -199,15 +199,21 @@ def test_release_thread_frees_the_scratch_and_later_calls_still_work(lib, oracle
         ok &= lib.w2v_release_thread() == 0          # a second release has nothing to free
         # and the thread can go on: scratch is allocated again
         ok &= lib.word2vecNeg(d, G, nwa, nwb, ptr(WAd), ptr(WBd), ptr(Ad), ptr(Bd), 0.005, 0.5) == 0
+        held2 = free0 - torch.cuda.mem_get_info()[0]
         ok &= lib.w2v_release_thread() == 0
-        result.update(ok=bool(ok), held=held, after=after)
+        after2 = free0 - torch.cuda.mem_get_info()[0]
+        result.update(ok=bool(ok), held=held, after=after, held2=held2, after2=after2)
 
     t = threading.Thread(target=worker)
     t.start()
     t.join()
     assert result["ok"]
-    assert result["held"] >= 8 << 20, result       # the thread's scratch was real device memory
-    assert result["after"] <= 2 << 20, result      # and the release gave it back
+    # the thread's scratch was real device memory and the release gave it back (what stays is
+    # what the runtime itself keeps after a first launch: code objects, queues); a second round
+    # of calls and release ends at the same level, so nothing accumulates
+    assert result["held"] - result["after"] >= 8 << 20, result
+    assert result["held2"] - result["after2"] >= 8 << 20, result
+    assert result["after2"] <= result["after"], result
     Ao, Bo = A.copy(), B.copy()
     oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.005, 0.5, 1)
     oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.005, 0.5, 1)

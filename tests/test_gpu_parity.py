@@ -98,6 +98,10 @@ def test_eval_pos_matches_oracle(gpu, oracle, d, V, N, skip):
     (100, 1000, 5000, 5, 5), (300, 5000, 6000, 5, 5), (512, 2000, 2000, 15, 5), (1, 10, 50, 1, 1),
     (64, 300, 500, 3, 2), (65, 300, 500, 7, 8), (1280, 200, 100, 5, 5), (50, 400, 300, 70, 4),
     (300, 500, 1000, 9, 1),
+    # more B words than one wave holds at once; (5, 10) is the reference GPU launcher's own shape
+    # (jni/src/DNN127.cu:1434)
+    (300, 5000, 2000, 5, 10), (100, 1000, 500, 3, 9), (512, 2000, 300, 15, 16), (64, 300, 200, 2, 64),
+    (1280, 200, 60, 5, 10), (30, 300, 200, 70, 21),
 ])
 def test_eval_neg_matches_oracle(gpu, oracle, d, V, G, nwa, nwb):
     rng = np.random.default_rng(d + G)
@@ -197,7 +201,10 @@ def test_pos_update_matches_oracle(gpu, oracle, vexp, d, skip, ncentres):
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 1.0, 0.75])
 @pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
                                          (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
-                                         (40, 70, 3, 40), (300, 6, 2, 100)])
+                                         (40, 70, 3, 40), (300, 6, 2, 100),
+                                         # nwb beyond the 8 columns a wave holds at once
+                                         (300, 5, 10, 200), (100, 5, 9, 100), (512, 15, 16, 40),
+                                         (64, 2, 64, 20), (1280, 5, 10, 20), (30, 70, 21, 10)])
 def test_neg_update_matches_oracle(gpu, oracle, vexp, d, nwa, nwb, G):
     rng = np.random.default_rng(d * 5 + nwa)
     V = 20000
@@ -292,7 +299,7 @@ def test_empty_and_rejected_arguments(gpu):
     assert CUMACH.word2vecPos(1281, 4, 5, I, I, I, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecPos(d, -1, 5, I, I, I, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecPos(d, 4, 5, None, I, I, A, B, 0.1, 0.5) == 1
-    assert CUMACH.word2vecNeg(d, 1, 5, 9, I, I, A, B, 0.1, 0.5) == 1
+    assert CUMACH.word2vecNeg(d, 1, 5, 65, I, I, A, B, 0.1, 0.5) == 1    # more B words than lanes
     assert CUMACH.word2vecNeg(d, 1, 5, 5, I, None, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecEvalPos(d, 4, 5, I, I, I, A, B, None) == 1
     assert CUMACH.word2vecEvalNeg(d, 1, 5, 5, I, I, A, None, ret) == 1

@@ -93,7 +93,9 @@ def test_pos_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols, 
 
 @pytest.mark.parametrize("islice,nslices,nhead,maxcols,dohead,dual", SLICINGS)
 @pytest.mark.parametrize("d,nwa,nwb,vexp", [(100, 5, 5, 0.0), (300, 15, 5, 0.5), (130, 3, 8, 0.5),
-                                            (64, 70, 2, 0.0)])
+                                            (64, 70, 2, 0.0),
+                                            # more B words than a wave holds at once
+                                            (300, 5, 10, 0.5), (100, 4, 21, 0.0)])
 def test_neg_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols, dohead, dual, d,
                                   nwa, nwb, vexp):
     torch, CUMACH = gpu
@@ -124,7 +126,8 @@ def test_eval_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols,
     from bidmach_amd.cumach import load_library
     lib = load_library()
     rng = np.random.default_rng(13 * d + islice)
-    V, N, skip, nwa, nwb, G = 3000, 20000, 5, 5, 5, 4000
+    V, N, skip, nwa, G = 3000, 20000, 5, 5, 4000
+    nwb = 5 if d == 100 else 10
     A, B = rand_tables(rng, V, d, 0.6 / math.sqrt(d) ** 0.5)
     W = corpus.zipf_stream(N, V, 1.0, seed=d + islice)
     W[rng.random(N) < 0.05] = -1
@@ -225,4 +228,4 @@ def test_bad_slice_arguments_are_rejected(gpu):
     assert pos([t[0]] * too_many) != 0
     assert CUMACH.word2vecEvalPosSlice(d, n, 2, W, W, W, t, 0, 1, 10, 0, 0, None) != 0
     assert CUMACH.word2vecEvalPosSlice(d, n, 2, W, W, W, t, 0, 1, 10, 0, 0, ret) == 0
-    assert CUMACH.word2vecNegSlice(d, 4, 2, 9, W, W, t, 0.1, 0.0, 0, 1, 10, 0, 0, 0) != 0  # nwb > 8
+    assert CUMACH.word2vecNegSlice(d, 4, 2, 65, W, W, t, 0.1, 0.0, 0, 1, 10, 0, 0, 0) != 0  # nwb > 64
