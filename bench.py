@@ -169,6 +169,11 @@ def main():
     ap.add_argument("--max-workgroups", type=int, default=0,
                     help="w2v_set_max_workgroups: bound on the workgroups of the update kernels "
                          "(0 = the whole device)")
+    ap.add_argument("--ordered-mode", type=int, default=-1, choices=(-1, 0, 1),
+                    help="w2v_set_ordered_mode: -1 the library's per-launch choice (default: "
+                         "launches full of frequent words run in the reference's order on a few "
+                         "hundred wavefronts), 0 never (throughput kernels whatever the stream), "
+                         "1 always")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -189,6 +194,7 @@ def main():
     from bidmach_amd.cumach import load_library
     load_library().w2v_set_hot_update_mode(args.hot_mode)
     load_library().w2v_set_rare_update_mode(args.rare_mode)
+    load_library().w2v_set_ordered_mode(args.ordered_mode)
     if args.bf16_hot_words >= 0:
         check(load_library().w2v_set_bf16_hot_words(args.bf16_hot_words), "w2v_set_bf16_hot_words")
     if args.max_workgroups > 0:
@@ -378,6 +384,8 @@ def main():
         out["config"]["hot_update_mode"] = args.hot_mode
     if args.rare_mode != -1:
         out["config"]["rare_update_mode"] = args.rare_mode
+    if args.ordered_mode != -1:
+        out["config"]["ordered_mode"] = args.ordered_mode
     if args.tokens > 0:
         out["roofline"]["traffic"] = None       # measured at the workload's own size only
     if args.wsample > 0.0:

@@ -536,6 +536,12 @@ int w2v_set_max_workgroups(int n) {
 }
 int w2v_get_max_workgroups(void) { return w2v::get_max_workgroups(); }
 
+int w2v_set_ordered_mode(int mode) {
+  w2v::set_ordered_mode(mode);
+  return 0;
+}
+int w2v_get_ordered_mode(void) { return w2v::get_ordered_mode(); }
+
 int w2v_set_rare_update_mode(int mode) {
   w2v::set_rare_update_mode(mode);
   return 0;

@@ -247,6 +247,9 @@ struct Shadow {
   float* pub_b;
   int* hot_mask;  // [2][kHotCountSlots] partial bit masks of the hot ids seen: table B's, then A's
   int xcc;        // the XCD this wave runs on (filled in by resolve_hot_mode)
+  // Ordered form of the update passes (see launch_is_ordered): 0 never, 1 when the device-side
+  // count finds the launch full of frequent words, 2 always.
+  int ordered;
 };
 
 constexpr int kOccurSlots = 1 << 20;
@@ -307,6 +310,25 @@ __device__ __forceinline__ int hot_mode_of(const Shadow& sh, int which) {
 __device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow& resolved) {
   return asked.hot_total > 0 && asked.combine != kHotOff && resolved.combine == kHotOff &&
          resolved.combine_a == kHotOff;
+}
+
+// Whether this launch runs in its ordered form.  A launch that is full of frequent words (a raw,
+// un-subsampled Zipf stream: a tenth of all tokens are word 0) trains at the edge of stability at
+// the reference's step size, and what its result then depends on is how many updates of the
+// frequent words' columns a reader misses.  The reference's CPU threads miss a handful (one pair
+// per thread in flight); thousands of work units in flight on a whole GPU miss thousands, and a
+// tile of adjacent tokens that shares one snapshot of its context columns misses every update
+// its own tokens make.  The held-out loss then lands many percent (or many hundred percent) away
+// from the reference's.  The ordered kernels (pos_chain_kernel, neg_rows_kernel) keep the
+// reference's order inside a worker - a wave walks its tokens / groups one after the other, reads
+// every column afresh and adds a B delta to the table before the next read - and keep the number
+// of workers at a few dozen, like a large multi-core host.  They run in place of the throughput
+// kernels, which return at once, when the count made on the device before the launch finds hot
+// words; launches without them (after frequent-word subsampling) keep the throughput kernels.
+__device__ __forceinline__ bool launch_is_ordered(const Shadow& asked, const Shadow& resolved) {
+  if (asked.ordered == 2) return true;
+  return asked.ordered == 1 && asked.hot_total > 0 &&
+         !(resolved.combine == kHotOff && resolved.combine_a == kHotOff);
 }
 
 __device__ __forceinline__ int shadow_copies(int w, int combine) {

@@ -103,6 +103,20 @@ hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int n
                                  const int* WA, const int* WB, const SliceMap& m, float lrate,
                                  float vexp);
 
+// Ordered form of the negative pass (w2v_neg_rows.hip), for launches whose device-side count
+// finds them full of frequent words: `chains` waves walk the groups row by row in the
+// reference's order.  It keeps the group's A columns in registers, so not every shape has an
+// instance (neg_rows_available).  Launched after the throughput kernel, which returns at once
+// when the launch is ordered, as this one does when it is not.
+bool neg_rows_available(int nrows, int nwa);
+hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                           const int* WA, const int* WB, float* A, float* B, float lrate,
+                           float vexp, int64_t chains, const Shadow& shadow);
+// Ordered form: -1 (default) chosen per launch on the device, 0 never, 1 always.
+void set_ordered_mode(int mode);
+int get_ordered_mode();
+int ordered_flag(bool forced_hot_mode);   // the value of Shadow::ordered for a launch
+
 // Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
 // and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or
 // Retval64[0] (double, added into).  Either output pointer may be null.

@@ -209,6 +209,141 @@ pos_eval_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ 
   block_store_partial(wave_sum_f64(lsum), partials);
 }
 
+// Ordered form of the update (launch_is_ordered, w2v_device.h): the token-by-token order of the
+// reference's CPU loop (BIDMach_CPUMACH.c:26-68).  A wave is one of a few dozen workers, like a
+// thread of the reference (:21-24): it walks a contiguous range of centre tokens one after the
+// other; for each it reads the centre's A column and the window's B columns afresh (device-scope
+// loads, so neither this CU's L1 nor this XCD's L2 can hand back a value from before another
+// worker's update), adds every B delta to the table at once and the A delta after the window,
+// and waits until those adds have been performed before it reads for the next token, whose
+// window shares all but two positions with this one.  (A tile of adjacent tokens that computes
+// from one snapshot of its columns misses exactly those updates: 16 tokens per snapshot move the
+// held-out loss of a raw Zipf stream by 5 %, 2 tokens by 1.7 %.)
+// The ids of the next token and of its window (offsets -32..31) are fetched while the current
+// token is worked on.
+constexpr int kChainLook = 32;
+template <int R, int CH>
+__global__ void __launch_bounds__(kBlock)
+pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
+                 const int* __restrict__ LB, const int* __restrict__ UB, float* A, float* B,
+                 float lrate, float vexp, int smode, Shadow shadow_arg) {
+  const Shadow shadow = resolve_hot_mode(shadow_arg);
+  if (!launch_is_ordered(shadow_arg, shadow)) return;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t chain = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t i_begin = chain * per_chain;
+  const int64_t i_end = min(i_begin + per_chain, (int64_t)ncols);
+
+  int lb = 0, ub = 0, wnear = -1;
+  auto fetch = [&](int64_t t) {
+    lb = ub = 0;
+    wnear = -1;
+    if (t < i_end) {
+      lb = LB[t];
+      ub = UB[t];
+      const int64_t p = t + lane - kChainLook;
+      if (p >= 0 && p < ncols) wnear = W[p];
+    }
+  };
+  fetch(i_begin);
+  for (int64_t unit = i_begin; unit < i_end; ++unit) {
+    const int i = (int)unit;
+    const int wi = read_lane(wnear, kChainLook);
+    const int jlo = max(__builtin_amdgcn_readfirstlane(lb), -i);
+    const int jhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 1 - i);
+    const int wnear_now = wnear;
+    fetch(unit + 1);
+    if (wi < 0) continue;
+    float* const acol = A + (int64_t)wi * d;
+    float a[R];
+    load_col_fresh<R>(a, acol, lane, d);
+    float daa[R];
+    zero_col<R>(daa);
+    const float ascale = scale_of(wi, vexp, smode);
+    bool touched = false;
+
+    const int base0 = min(jlo, -kChainLook);
+    for (int base = base0; base <= jhi; base += kWave) {
+      // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand.
+      // (A window wider than 64 offsets is worked on in slabs, each after the adds of the last.)
+      if (base != base0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      const int j = base + lane;
+      int wl = -1;
+      if (j >= jlo && j <= jhi && j != 0)
+        wl = base == -kChainLook ? wnear_now : W[i + j];
+      const bool ok = wl >= 0;
+      const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
+      const unsigned long long valid = __ballot(ok);
+      // A word that stands at several offsets of the window is updated once per offset, and the
+      // reference reads it again each time (:43-46 after :60): occurrence number r of a word is
+      // worked on in round r, after the adds of round r - 1 have been performed.  Pairs of
+      // different words commute, so the rounds change nothing else.
+      int occ = 0;
+      {
+        unsigned long long m = valid;
+        while (m != 0ull) {
+          const int l = __builtin_ctzll(m);
+          m &= m - 1ull;
+          if (l < lane && read_lane(wl, l) == wl) ++occ;
+        }
+      }
+      for (int round = 0;; ++round) {
+        unsigned long long mask = __ballot(ok && occ == round);
+        if (mask == 0ull) break;
+        if (round > 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        while (mask != 0ull) {
+          int src[CH];
+          int n = 0;
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (mask != 0ull) {
+              src[c] = __builtin_ctzll(mask);
+              mask &= mask - 1ull;
+              n = c + 1;
+            } else {
+              src[c] = -1;
+            }
+          }
+          float b[CH][R];
+          int wb[CH];
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (c < n) {
+              wb[c] = read_lane(wl, src[c]);
+              load_col_fresh<R>(b[c], B + (int64_t)wb[c] * d, lane, d);
+            }
+          }
+          float pre = 0.0f;
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (c < n) {
+              const float s = wave_sum(dot_partial<R>(a, b[c]));
+              pre = (lane == c) ? s : pre;
+            }
+          }
+          const float gl = lrate * (1.0f - sat_sigmoid(pre));
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (c < n) {
+              const float g = read_lane(gl, c);
+              const float bs = read_lane(sl, src[c]);
+              axpy<R>(daa, ascale * g, b[c]);
+              atomic_axpy_col<R>(B + (int64_t)wb[c] * d, bs * g, a, lane, d);
+            }
+          }
+          touched = true;
+        }
+      }
+    }
+    if (touched) {
+      atomic_add_col<R>(acol, daa, lane, d);
+      // the adds of this token are performed before the next token's columns are read
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    }
+  }
+}
+
 constexpr int64_t kMinEvalCentresPerWg = 256;
 
 constexpr int kTileWaves = 8;
@@ -263,6 +398,7 @@ pos_tile_kernel(int d, int ncols, int T, int Sh, int carry, int64_t ntiles,
   float* const pend = reinterpret_cast<float*>(ft + (T + 2 * Sh));
   const int slot = blockIdx.x;  // picks the shadow copy this workgroup writes to
 
+  if (launch_is_ordered(shadow_arg, shadow)) return;   // pos_chain_kernel does this launch
   const bool cold = launch_is_cold(shadow_arg, shadow);
   const int64_t tiles_per_wg = cold ? tiles_per_wg_wide : tiles_per_wg_hot;
   // Measured: handing deltas on pays on launches without hot words (6 % on a subsampled stream),
@@ -624,6 +760,16 @@ static std::atomic<int> g_max_workgroups{0};
 void set_max_workgroups(int n) { g_max_workgroups.store(n < 0 ? 0 : n); }
 int get_max_workgroups() { return g_max_workgroups.load(); }
 
+static std::atomic<int> g_ordered_mode{-1};
+void set_ordered_mode(int mode) { g_ordered_mode.store(mode == 0 || mode == 1 ? mode : -1); }
+int get_ordered_mode() { return g_ordered_mode.load(); }
+int ordered_flag(bool forced_hot_mode) {
+  const int mode = g_ordered_mode.load();
+  if (mode == 1) return 2;
+  if (mode == 0 || forced_hot_mode) return 0;   // a forced hot-word mode asks for that mode
+  return 1;
+}
+
 static std::atomic<int> g_hot_update_mode{-1};
 void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode >= 0 && mode <= 2 ? mode : -1); }
 int get_hot_update_mode() { return g_hot_update_mode.load(); }
@@ -649,6 +795,7 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   else
     shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
   shadow->combine_a = shadow->combine;
+  shadow->ordered = Tables::kSliced ? 0 : ordered_flag(forced);
   if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
   if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
@@ -789,6 +936,30 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
   return hipGetLastError();
 }
 
+// Workers of the ordered form: as many as keep the missed updates of the most frequent word near
+// what a few dozen CPU threads miss (a lockstep simulation of K workers lands 0.2 %, 0.6 %, 1.4 %,
+// 5 % from the sequential result at K = 16, 32, 128, 256 on a raw Zipf stream), and no fewer
+// than 64 tokens per worker.
+constexpr int kPosChains = 128;
+constexpr int64_t kMinTokensPerChain = 64;
+
+template <int R>
+static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, const int* W,
+                                   const int* LB, const int* UB, float* A, float* B, float lrate,
+                                   float vexp, const Shadow& shadow) {
+  int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
+  if (chains > kPosChains) chains = kPosChains;
+  const int limit = g_max_workgroups.load();
+  if (limit > 0 && chains > (int64_t)limit * kWavesPerBlock) chains = (int64_t)limit * kWavesPerBlock;
+  if (chains < 1) chains = 1;
+  const int64_t per_chain = ((int64_t)ncols + chains - 1) / chains;   // waves beyond: empty range
+  hipLaunchKernelGGL((pos_chain_kernel<R, PosChunk<R>::value>),
+                     dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
+                     dim3(kBlock), 0, stream, d, ncols, per_chain, W, LB, UB, A, B, lrate, vexp,
+                     scale_mode(vexp), shadow);
+  return hipGetLastError();
+}
+
 // Tile size: 16 tokens, or 8 if that is what lets two workgroups share a CU's LDS; if even 8
 // tokens do not fit in one CU's LDS the per-centre kernel is used instead.  A tile is a small
 // synchronous batch (all its dot products use the staged columns), so larger tiles would trade
@@ -844,6 +1015,13 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
                      scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
+  if constexpr (!Tables::kSliced) {
+    if (shadow.ordered != 0) {
+      err = launch_pos_chain<R>(stream, d, ncols, W, LB, UB, tables.A, tables.B, lrate, vexp,
+                                shadow);
+      if (err != hipSuccess) return err;
+    }
+  }
   return launch_fold(stream, fold_a, fold_b, shadow, d);
 }
 

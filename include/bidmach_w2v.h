@@ -189,6 +189,26 @@ int w2v_release_thread(void);
 int w2v_set_max_workgroups(int n);
 int w2v_get_max_workgroups(void);
 
+/* Ordered form of word2vecPos / word2vecNeg / word2vecNegFilt, process-wide.  The reference's CPU
+ * path keeps as many work units in flight as it has threads (BIDMach_CPUMACH.c:21-24, :197-201),
+ * each of which reads a column just before it uses it and writes a B column back before it
+ * reads the next (:57-61, :244-246).  On a raw (not subsampled) Zipf stream, where a tenth of
+ * all tokens are the most frequent word, training at the reference's step size is at the edge
+ * of stability and its result depends on how many updates of the frequent words a reader
+ * misses; thousands of work units in flight, or a tile of adjacent tokens working from one
+ * snapshot, then end many percent away from the reference's held-out loss.  In the ordered form
+ * a few hundred wavefronts each walk a contiguous range of tokens / groups in the reference's
+ * order, with every column read afresh and every B delta added before the next read.
+ *  -1  (default) decided per launch on the device, by the same count that decides about shadow
+ *      copies below: ordered if at least 1/16 of the word ids of the launch are among the 16
+ *      lowest, or at least 1/48 are id 0; launches without frequent words (after the reference
+ *      caller's subsampling, Word2Vec.scala:221-225) keep the throughput kernels.  A forced
+ *      w2v_set_hot_update_mode also keeps them.
+ *   0  never;  1  always.
+ * Sliced models and groups with more than 8 B words always use the throughput kernels. */
+int w2v_set_ordered_mode(int mode);
+int w2v_get_ordered_mode(void);
+
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
  * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
  *   0  exact: their atomics are spread over shadow copies and every reader sums the copies;

@@ -1,0 +1,153 @@
+"""The ordered form of the update operators (w2v_set_ordered_mode in include/bidmach_w2v.h): the
+kernels that walk tokens / groups in the reference's order on a bounded number of workers, taken
+by default for launches full of frequent words.  (needs an MI355X)
+
+Forced on, they must pass the same oracle checks as the throughput kernels.  What sets them apart
+is checked on minibatches made of a handful of words, where every update collides with the ones
+before it: a launch small enough for one worker must then reproduce the oracle's SEQUENTIAL
+result (jni/src/BIDMach_CPUMACH.c:26-68, :210-254 at one thread), which no kernel that works
+from a snapshot of its columns can.
+"""
+import numpy as np
+import pytest
+
+from bidmach_amd import corpus
+from tests import test_gpu_parity as parity
+
+pytestmark = pytest.mark.gpu
+
+gpu = parity.gpu
+
+
+@pytest.fixture
+def ordered():
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    assert lib.w2v_get_ordered_mode() == -1
+    lib.w2v_set_ordered_mode(1)
+    yield lib
+    lib.w2v_set_ordered_mode(-1)
+
+
+@pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
+@pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (512, 10, 100),
+                                             (1, 2, 50), (65, 3, 100), (1280, 5, 40),
+                                             (24, 40, 30)])
+def test_pos_update_forced_ordered(gpu, oracle, ordered, vexp, d, skip, ncentres):
+    parity.test_pos_update_matches_oracle(gpu, oracle, vexp, d, skip, ncentres)
+
+
+@pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
+@pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
+                                         (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
+                                         (40, 70, 3, 40), (300, 6, 2, 100), (640, 16, 4, 50),
+                                         (700, 6, 5, 50)])
+def test_neg_update_forced_ordered(gpu, oracle, ordered, vexp, d, nwa, nwb, G):
+    # (40, 70, 3) and (700, 6, 5) have no row-by-row instance: the group-at-a-time kernel on a
+    # few workgroups stands in
+    parity.test_neg_update_matches_oracle(gpu, oracle, vexp, d, nwa, nwb, G)
+
+
+def test_other_checks_forced_ordered(gpu, oracle, ordered):
+    parity.test_pos_update_ragged_windows_and_tile_edges(gpu, oracle)
+    parity.test_neg_filt_matches_oracle(gpu, oracle, 100, 10, 5)
+    parity.test_neg_filt_matches_oracle(gpu, oracle, 300, 5, 5)
+    parity.test_heavy_collisions_lose_no_contribution(gpu)
+    parity.test_noop_invariants_on_gpu(gpu)
+    for shift in (0, 2, 100):
+        parity.test_pos_update_any_shift_argument(gpu, oracle, shift)
+
+
+def tiny_colliding(rng, d, V, n, skip):
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    W = rng.integers(0, V, n).astype(np.int32)
+    W[rng.random(n) < 0.1] = -1
+    LB, UB = corpus.window_bounds(n, skip, rng)
+    return A, B, W, LB, UB
+
+
+@pytest.mark.parametrize("d,skip", [(100, 5), (300, 3), (64, 12)])
+def test_one_worker_reproduces_the_sequential_positive_pass(gpu, oracle, d, skip):
+    """60 tokens over 6 words: every pair updates columns the pairs before it updated.  The
+    launch holds only frequent words (ids below 16), so the default takes the ordered form, and
+    60 tokens are one worker's range: the result is the oracle's one-thread result up to the
+    rounding of the dot products.  The throughput kernel (ordered form off) works from one
+    snapshot per tile and lands visibly elsewhere."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(d)
+    A, B, W, LB, UB = tiny_colliding(rng, d, 6, 60, skip)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecPos(d, 60, skip, W, LB, UB, Ao, Bo, 0.05, 0.5, 1)
+    Ag, Bg = parity.gpu_pos(gpu, d, skip, W, LB, UB, A, B, 0.05, 0.5)
+    err = max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max())
+    assert err <= 2e-5, err
+    lib.w2v_set_ordered_mode(0)
+    try:
+        At, Bt = parity.gpu_pos(gpu, d, skip, W, LB, UB, A, B, 0.05, 0.5)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+    assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
+
+
+@pytest.mark.parametrize("d,nwa,nwb", [(100, 5, 5), (300, 5, 5), (200, 12, 3)])
+def test_one_worker_reproduces_the_sequential_negative_pass(gpu, oracle, d, nwa, nwb):
+    """16 groups over 8 words (distinct inside a group's B words and inside its A words, as the
+    group-level order of the reference matters only there): B columns change from row to row and
+    from group to group, A columns from group to group."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(d + nwa)
+    V, G = 14, 16
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    WA = np.concatenate([rng.permutation(V)[:nwa] for _ in range(G)]).astype(np.int32)
+    WB = np.concatenate([rng.permutation(V)[:nwb] for _ in range(G)]).astype(np.int32)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.05, 0.5, 1)
+    Ag, Bg = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, 0.05, 0.5)
+    err = max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max())
+    assert err <= 2e-5, err
+    lib.w2v_set_ordered_mode(0)
+    try:
+        At, Bt = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, 0.05, 0.5)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+    assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
+
+
+def test_a_word_twice_among_a_groups_b_words_sees_its_first_update(gpu, oracle):
+    """The reference writes a B column back before it turns to the next B word (:244-246), so a
+    word that is a group's B word twice is dotted the second time with its first delta in it."""
+    rng = np.random.default_rng(11)
+    d, V, G, nwa, nwb = 100, 14, 8, 5, 5
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    WA = np.concatenate([rng.permutation(V)[:nwa] for _ in range(G)]).astype(np.int32)
+    WB = np.concatenate([rng.permutation(V)[:nwb] for _ in range(G)]).astype(np.int32)
+    WB[1::nwb] = WB[0::nwb]          # rows 0 and 1 of every group are the same word
+    WB[4::nwb] = WB[2::nwb]          # and rows 2 and 4
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.05, 0.0, 1)
+    Ag, Bg = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, 0.05, 0.0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
+
+
+def test_launches_without_frequent_words_keep_the_throughput_kernels(gpu, oracle):
+    """The decision is made on the device from the ids of the launch: with no id below 16 the
+    ordered kernels return at once, whatever the collisions (here: the same heavy collisions on
+    ids 100..105, where the tile's snapshot semantics show)."""
+    rng = np.random.default_rng(5)
+    d, skip = 100, 5
+    A, B, W, LB, UB = tiny_colliding(rng, d, 6, 60, skip)
+    big = np.zeros((200, d), np.float32)
+    A2, B2 = big.copy(), big.copy()
+    A2[100:106], B2[100:106] = A, B
+    W2 = np.where(W >= 0, W + 100, -1).astype(np.int32)
+    Ao, Bo = A2.copy(), B2.copy()
+    oracle.word2vecPos(d, 60, skip, W2, LB, UB, Ao, Bo, 0.05, 0.0, 1)
+    Ag, Bg = parity.gpu_pos(gpu, d, skip, W2, LB, UB, A2, B2, 0.05, 0.0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) > 1e-3

@@ -9,12 +9,16 @@ index arrays and initial tables.  The score is the reference's (Word2Vec.scala:2
 Two regimes:
   "subsampled"  the reference caller's default frequent-word subsampling, wsample = 1e-4
                 (Word2Vec.scala:150,221-225,579).  Tolerance 0.5 %.
-  "raw"         no subsampling: 10 % of all tokens are word 0.  In this regime the loss of a
-                sequential run is set by how finely the updates of the few hottest columns
-                interleave; the CPU oracle itself moves by 0.3-0.4 % between 1 and 8 threads, and
-                any implementation that keeps more than a few hundred tokens in flight lands
-                several percent away (lower).  The test checks that training stays finite and
-                reports the distance; it asserts only a loose band.
+  "raw"         no subsampling, as the configuration is written: 10 % of all tokens are word 0 and
+                training at lr 0.025 is at the edge of stability (the sequential run ends ABOVE
+                the untrained loss).  The loss is then set by how many updates of the frequent
+                words a reader misses, and the oracle itself moves by up to a percent with its
+                thread count, from run to run (on a 16-core host: +1.1 % at 8 threads, +2.8 % at 16).
+                The library takes its ordered kernels for such
+                launches by itself (w2v_set_ordered_mode, default); the test runs it with default
+                settings on the whole device and asserts the band
+                    max over T in {2, 4, 8, 16} of |oracle(T threads) / oracle(1 thread) - 1| + 0.5 %
+                derived in the same run, twice (no run-to-run blow-up).
 """
 import numpy as np
 import pytest
@@ -97,28 +101,106 @@ def test_heldout_loss_subsampled_within_half_percent(oracle):
     assert abs(gpu - cpu_seq) <= 0.005 * cpu_seq, (gpu, cpu_seq)
 
 
-def test_heldout_loss_raw_stream_bounded_run_stays_close(oracle):
+def oracle_band(runs, seq):
+    """Largest relative distance of the multi-threaded oracle runs from the sequential one, plus
+    the half percent of the tolerance."""
+    return max(abs(r / seq - 1.0) for r in runs) + 0.005
+
+
+def test_heldout_loss_raw_stream_default_settings_within_the_oracles_own_band(oracle):
     from bidmach_amd.cumach import load_library
     lib = load_library()
+    assert lib.w2v_get_ordered_mode() == -1 and lib.w2v_get_max_workgroups() == 0
+    assert lib.w2v_get_hot_update_mode() == -1 and lib.w2v_get_rare_update_mode() == -1
     stream = make_stream(0.0)
     cpu_seq = cpu_run(oracle, stream, 1)
-    cpu_par = cpu_run(oracle, stream, 8)
-    gpu = gpu_run(stream)
+    cpu_par = {t: cpu_run(oracle, stream, t) for t in (2, 4, 8, 16)}
+    band = oracle_band(cpu_par.values(), cpu_seq)
+    gpu = [gpu_run(stream) for _ in range(2)]
+    print("\nraw: held-out loss cpu(1 thread) %.5f; cpu(T threads) %s; band %.3f%%; "
+          "gpu, default settings, two runs: %s"
+          % (cpu_seq, ", ".join("T=%d %+.3f%%" % (t, 100.0 * (v / cpu_seq - 1.0))
+                                for t, v in cpu_par.items()), 100.0 * band,
+             ", ".join("%.5f (%+.3f%%)" % (g, 100.0 * (g / cpu_seq - 1.0)) for g in gpu)))
+    assert 0.005 <= band <= 0.10, band            # the oracle's own spread: a few percent at most
+    for g in gpu:
+        assert np.isfinite(g)
+        assert abs(g / cpu_seq - 1.0) <= band, (g, cpu_seq, band)
+    # for the record: the throughput kernels on the same stream (what the default avoids)
     try:
-        lib.w2v_set_max_workgroups(8)      # 8 ordered streams, like 8 CPU threads
-        gpu8 = gpu_run(stream)
+        lib.w2v_set_ordered_mode(0)
+        fast = gpu_run(stream)
     finally:
-        lib.w2v_set_max_workgroups(0)
-    print("\nraw: held-out loss cpu(1 thread) %.5f cpu(8 threads) %.5f (%+.3f%%) "
-          "gpu %.5f (%+.3f%%) gpu limited to 8 workgroups %.5f (%+.3f%%)"
-          % (cpu_seq, cpu_par, 100.0 * (cpu_par / cpu_seq - 1.0), gpu,
-             100.0 * (gpu / cpu_seq - 1.0), gpu8, 100.0 * (gpu8 / cpu_seq - 1.0)))
-    # With a tenth of all tokens being word 0 and hundreds of groups in flight, the whole-device
-    # run is at the edge of stability at this step size: its loss moves by large factors from run
-    # to run (the 8-thread CPU run moves by a percent as well), so it is only reported; the run
-    # bounded to 8 workgroups is stable and must stay near the CPU runs.
-    assert np.isfinite(gpu8)
-    assert abs(gpu8 - cpu_seq) <= 0.2 * cpu_seq, (gpu8, cpu_seq)
+        lib.w2v_set_ordered_mode(-1)
+    print("raw: throughput kernels forced (w2v_set_ordered_mode(0)): %.5f (%+.1f%%)"
+          % (fast, 100.0 * (fast / cpu_seq - 1.0)))
+
+
+def test_headline_shape_raw_stream_default_settings_within_the_oracles_own_band(oracle):
+    """The headline shape as the configuration states it (vocab 1M, dim 300, 1M-token minibatches
+    of the raw Zipf stream), 8 minibatches.  A sequential oracle run of this size takes minutes,
+    so the band is derived from the oracle's 16-thread runs against its 8-thread run (the same
+    run-to-run and thread-count spread, measured where it is affordable), plus 0.5 %; the GPU,
+    with default settings, must be within it of the 8-thread run.  At this step size the loss of
+    every run is far above the untrained 1.386: this regime does not train, on the CPU either,
+    and what is compared is how it fails."""
+    import torch
+    from bidmach_amd.cumach import CUMACH, check
+    Vh, Dh, Nh, K = 1_000_000, 300, 1_000_000, 8
+    zc = corpus.zipf_cdf(Vh, 1.0)
+    nc = corpus.unigram_pow_cdf(Vh, 1.0, 0.75)
+
+    def mb(i):
+        W = corpus.zipf_stream(Nh, Vh, 1.0, seed=1234 + i, cdf=zc)
+        rng = np.random.Generator(np.random.PCG64(99 + i))
+        LB, UB = corpus.window_bounds(Nh, SKIP, rng)
+        WA, WB, G = corpus.negative_groups(W, LB, UB, NNEG, NREUSE, rng, neg_cdf=nc)
+        return W, LB, UB, WA, WB, G
+
+    def lr(i):
+        return max(LR0 * (1.0 - i / K), LR0 * 1e-4)
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    mbs = [mb(i) for i in range(K + 1)]
+
+    def heldout(A, B):
+        W, LB, UB, WA, WB, G = mbs[K]
+        epos = oracle.word2vecEvalPos(Dh, Nh, SKIP, W, LB, UB, A, B, 16)
+        eneg = oracle.word2vecEvalNeg(Dh, G, NNEG, NREUSE, WA, WB, A, B, 16)
+        return -(epos + eneg / NNEG) / (G * NREUSE)
+
+    def cpu(nt):
+        B, A = corpus.init_tables(Vh, Dh, 42)
+        for i in range(K):
+            W, LB, UB, WA, WB, G = mbs[i]
+            oracle.word2vecPos(Dh, Nh, SKIP, W, LB, UB, A, B, lr(i), 0.0, nt)
+            oracle.word2vecNeg(Dh, G, NNEG, NREUSE, WA, WB, A, B, lr(i) / NNEG, 0.0, nt)
+        return heldout(A, B)
+
+    def gpu():
+        B, A = corpus.init_tables(Vh, Dh, 42)
+        Ad, Bd = dev(A), dev(B)
+        for i in range(K):
+            W, LB, UB, WA, WB, G = mbs[i]
+            check(CUMACH.word2vecPos(Dh, Nh, SKIP, dev(W), dev(LB), dev(UB), Ad, Bd, lr(i), 0.0),
+                  "pos")
+            check(CUMACH.word2vecNeg(Dh, G, NNEG, NREUSE, dev(WA), dev(WB), Ad, Bd,
+                                     lr(i) / NNEG, 0.0), "neg")
+        return heldout(Ad.cpu().numpy(), Bd.cpu().numpy())
+
+    ref = cpu(8)
+    par = [cpu(16), cpu(16)]
+    band = oracle_band(par, ref)
+    got = [gpu(), gpu()]
+    print("\nheadline shape, raw: held-out loss cpu(8 threads) %.5f; cpu(16 threads) %s; band "
+          "%.2f%%; gpu, default settings, two runs: %s"
+          % (ref, ", ".join("%.5f" % v for v in par), 100.0 * band,
+             ", ".join("%.5f (%+.2f%%)" % (g, 100.0 * (g / ref - 1.0)) for g in got)))
+    for g in got:
+        assert np.isfinite(g)
+        assert abs(g / ref - 1.0) <= band, (g, ref, band)
 
 
 def test_headline_shape_subsampled_loss_and_full_size_eval(oracle):
