@@ -541,6 +541,11 @@ int w2v_set_ordered_mode(int mode) {
   return 0;
 }
 int w2v_get_ordered_mode(void) { return w2v::get_ordered_mode(); }
+int w2v_set_ordered_workers(int pos_workers, int neg_workers) {
+  if (pos_workers < 0 || neg_workers < 0) return (int)hipErrorInvalidValue;
+  w2v::set_ordered_workers(pos_workers, neg_workers);
+  return 0;
+}
 
 int w2v_set_rare_update_mode(int mode) {
   w2v::set_rare_update_mode(mode);

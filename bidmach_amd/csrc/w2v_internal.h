@@ -116,6 +116,10 @@ hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit
 void set_ordered_mode(int mode);
 int get_ordered_mode();
 int ordered_flag(bool forced_hot_mode);   // the value of Shadow::ordered for a launch
+// Workers (wavefronts) of the ordered kernels; 0 = the built-in numbers.
+void set_ordered_workers(int pos, int neg);
+int ordered_pos_workers();
+int ordered_neg_workers();
 
 // Eval launchers write one double per block into `partials` (capacity >= eval_partials_needed)
 // and then fold them, in a fixed order, into Retval32[0] (float, added into) and/or

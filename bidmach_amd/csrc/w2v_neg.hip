@@ -447,7 +447,7 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   // ordered launches: the row-by-row kernel where it has an instance for the shape, else this
   // kernel on a few workgroups
   const bool rows = shadow.ordered != 0 && neg_rows_available(d, nwa);
-  int64_t chains = kNegChains;
+  int64_t chains = ordered_neg_workers() > 0 ? ordered_neg_workers() : kNegChains;
   const int limit = get_max_workgroups();
   if (limit > 0 && chains > (int64_t)limit * kNegWaves) chains = (int64_t)limit * kNegWaves;
   int64_t per_wg_ordered = 0;

@@ -770,6 +770,14 @@ int ordered_flag(bool forced_hot_mode) {
   return 1;
 }
 
+static std::atomic<int> g_ordered_pos_workers{0}, g_ordered_neg_workers{0};
+void set_ordered_workers(int pos, int neg) {
+  g_ordered_pos_workers.store(pos > 0 ? pos : 0);
+  g_ordered_neg_workers.store(neg > 0 ? neg : 0);
+}
+int ordered_pos_workers() { return g_ordered_pos_workers.load(); }
+int ordered_neg_workers() { return g_ordered_neg_workers.load(); }
+
 static std::atomic<int> g_hot_update_mode{-1};
 void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode >= 0 && mode <= 2 ? mode : -1); }
 int get_hot_update_mode() { return g_hot_update_mode.load(); }
@@ -948,7 +956,8 @@ static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, const i
                                    const int* LB, const int* UB, float* A, float* B, float lrate,
                                    float vexp, const Shadow& shadow) {
   int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
-  if (chains > kPosChains) chains = kPosChains;
+  const int64_t most = ordered_pos_workers() > 0 ? ordered_pos_workers() : kPosChains;
+  if (chains > most) chains = most;
   const int limit = g_max_workgroups.load();
   if (limit > 0 && chains > (int64_t)limit * kWavesPerBlock) chains = (int64_t)limit * kWavesPerBlock;
   if (chains < 1) chains = 1;

@@ -208,6 +208,10 @@ int w2v_get_max_workgroups(void);
  * Sliced models and groups with more than 8 B words always use the throughput kernels. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
+/* Number of wavefronts (workers) the ordered form of word2vecPos and of word2vecNeg / NegFilt
+ * spreads a launch over; 0 = the library's own numbers (the default).  Fewer workers follow the
+ * sequential order more closely and take longer; w2v_set_max_workgroups bounds them as well. */
+int w2v_set_ordered_workers(int pos_workers, int neg_workers);
 
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
  * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
