@@ -155,9 +155,10 @@ def parse_args():
                          "this process is worker 0 and holds only its share of the model")
     ap.add_argument("--head", type=int, default=0,
                     help="with --parts: number of head words (resident on every worker)")
-    ap.add_argument("--rare-mode", type=int, default=-1, choices=(-1, 0, 1),
+    ap.add_argument("--rare-mode", type=int, default=-1,
                     help="w2v_set_rare_update_mode: 0 = float atomics for every column, -1/1 = "
-                         "plain read-modify-write for words that are rare within a call (default)")
+                         "plain read-modify-write for words that are rare within a call "
+                         "(default), n >= 2 = for words with at most n occurrences in the call")
     ap.add_argument("--tokens", type=int, default=0,
                     help="tokens per minibatch, overriding the workload's (the reference's own "
                          "default minibatch is 100000 tokens)")
