@@ -307,6 +307,40 @@ struct Timer {
   hipEvent_t stop;
 };
 
+// ---- the entry point that allocates nothing ------------------------------------------------
+//
+// word2vecEvalNeg's kernels leave one partial sum per workgroup in a scratch buffer that a second
+// kernel folds; the ordinary entry point takes that buffer from hipMalloc on a thread's first
+// call.  word2vecEvalNegNoAlloc uses this array instead: device memory that is part of the loaded
+// code object, 64 KB on every GPU the library runs on, for the life of the process.
+constexpr int64_t kStaticPartials = 8192;
+constexpr int kNoAllocMaxGroups = 1 << 24;
+static __device__ __align__(256) double scratch[kStaticPartials];
+
+// The array's device address, per device (each GPU holds its own copy at its own address).  In
+// host code the name `scratch` is only a handle for hipGetSymbolAddress, never an address.
+std::atomic<double*> g_scratch_ptr[kMaxDevices];
+
+hipError_t static_scratch(double** out) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  double* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    // first call on this device, which is current: look the address up (threads that race here
+    // all get the same answer)
+    void* addr = nullptr;
+    err = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (addr == nullptr) return hipErrorInvalidSymbol;
+    p = static_cast<double*>(addr);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" {
@@ -367,6 +401,26 @@ int word2vecEvalNeg(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, fl
                     float* Retval) {
   return eval_neg_impl(nrows, ncols, nwa, nwb, WA, WB, A, B, Retval, nullptr, true);
 }
+
+int word2vecEvalNegNoAlloc(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A,
+                           float* B, float* Retval) {
+  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || !Retval)
+    return (int)hipErrorInvalidValue;
+  if (ncols > kNoAllocMaxGroups) return (int)hipErrorInvalidValue;   // beyond the stated maximum
+  if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
+  if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  double* partials = nullptr;
+  hipError_t err = static_scratch(&partials);
+  if (err != hipSuccess) return (int)err;
+  // every workgroup overwrites its own partial sum and the fold reads only those: nothing in
+  // the array has to start at zero
+  return finish(w2v::launch_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+                                     g_eval_floor.load(), partials, Retval, nullptr,
+                                     kStaticPartials),
+                true);
+}
+
+int w2v_no_alloc_max_groups(void) { return kNoAllocMaxGroups; }
 
 int word2vecEvalPosF64(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A,
                        float* B, double* Retval) {

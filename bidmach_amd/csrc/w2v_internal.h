@@ -128,9 +128,11 @@ hipError_t launch_eval_pos(hipStream_t stream, int nrows, int ncols, const int* 
                            const int* UB, const float* A, const float* B, double floorv,
                            double* partials, float* Retval32, double* Retval64);
 
+// partials_capacity: doubles `partials` holds, if fewer than eval_partials_needed (0: that many).
 hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, const float* A, const float* B,
-                           double floorv, double* partials, float* Retval32, double* Retval64);
+                           double floorv, double* partials, float* Retval32, double* Retval64,
+                           int64_t partials_capacity = 0);
 
 hipError_t launch_finalize(hipStream_t stream, double* partials, int64_t n, float* Retval32,
                            double* Retval64);

@@ -414,7 +414,8 @@ static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, ngroups,
                                    kMinEvalGroupsPerWg, &nwg);
   if (err != hipSuccess) return err;
-  const int64_t cap = eval_partials_needed(ngroups);   // what the caller's buffer holds
+  int64_t cap = eval_partials_needed(ngroups);   // what the caller's buffer holds,
+  if (*nparts > 0 && *nparts < cap) cap = *nparts;   // unless the caller says it holds less
   if (nwg > cap) nwg = cap;
   const int64_t groups_per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + groups_per_wg - 1) / groups_per_wg;
@@ -503,10 +504,11 @@ hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int
 
 hipError_t launch_eval_neg(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, const float* A, const float* B,
-                           double floorv, double* partials, float* Retval32, double* Retval64) {
+                           double floorv, double* partials, float* Retval32, double* Retval64,
+                           int64_t partials_capacity) {
   const int rounds = (nrows + kWave - 1) / kWave;
   hipError_t err = hipSuccess;
-  int64_t nparts = 0;
+  int64_t nparts = partials_capacity;   // in: capacity of `partials` (0: the default), out: used
 #define CALL(R)                                                                                   \
   err = launch_neg_r<R, false>(stream, nrows, ncols, 0, nwa, nwb, WA, WB, const_cast<float*>(A),  \
                                const_cast<float*>(B), 0.0f, 0.0f, floorv, partials, &nparts,      \

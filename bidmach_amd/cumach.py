@@ -48,6 +48,8 @@ SYMBOLS = {
     "word2vecEvalNeg": (_I, _ENEG),
     "word2vecEvalPosF64": (_I, _EPOS),
     "word2vecEvalNegF64": (_I, _ENEG),
+    "word2vecEvalNegNoAlloc": (_I, _ENEG),
+    "w2v_no_alloc_max_groups": (_I, []),
     "word2vecPosAsync": (_I, _POS),
     "word2vecNegAsync": (_I, _NEG),
     "word2vecEvalPosAsync": (_I, _EPOS),

@@ -105,6 +105,20 @@ int word2vecEvalPosF64(int nrows, int ncols, int shift, int *W, int *LB, int *UB
 int word2vecEvalNegF64(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
                        float *B, double *Retval);
 
+/* word2vecEvalNeg for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and the same result as word2vecEvalNeg (added into the device float Retval[0];
+ * blocking), but the per-workgroup partial sums go to a 64 KB array that is part of the library's
+ * device code instead of a buffer taken from hipMalloc on a thread's first call, and the call
+ * makes no hipMalloc, hipFree or other allocating call.  At most w2v_no_alloc_max_groups()
+ * (16,777,216) groups per call; more is rejected with hipErrorInvalidValue.  Every call on a GPU
+ * uses that GPU's one array: calls that overlap in time on one GPU (from several threads or
+ * streams) race and return wrong sums; one after the other they are independent (nothing in the
+ * array carries over). */
+int word2vecEvalNegNoAlloc(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
+                           float *B, float *Retval);
+int w2v_no_alloc_max_groups(void);
+
 /* Enqueue-only forms of the four operators: same arguments, same results, but they return after
  * the launch; completion is observed with w2v_synchronize() or a timer. */
 int word2vecPosAsync(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float *A, float *B,
