@@ -30,6 +30,7 @@
 // A token therefore costs about (2T + 2Sh)/T columns of atomics instead of 1 + (pairs).
 // All dot products of a tile use the columns as staged (a tile is a small synchronous batch);
 // between tiles the updates are Hogwild, as between the reference's threads.
+#include <algorithm>
 #include <atomic>
 
 #include "w2v_device.h"
@@ -952,11 +953,15 @@ constexpr int kPosChains = 128;
 constexpr int64_t kMinTokensPerChain = 64;
 
 template <int R>
-static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, const int* W,
+static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shift, const int* W,
                                    const int* LB, const int* UB, float* A, float* B, float lrate,
                                    float vexp, const Shadow& shadow) {
   int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
-  const int64_t most = ordered_pos_workers() > 0 ? ordered_pos_workers() : kPosChains;
+  // what is bounded is the pairs in flight: a token of a window of half-width 10 has twice the
+  // pairs of one of half-width 5, so half the workers
+  int64_t builtin = kPosChains;
+  if (shift > 5) builtin = std::max<int64_t>(32, kPosChains * 6 / (shift + 1));
+  const int64_t most = ordered_pos_workers() > 0 ? ordered_pos_workers() : builtin;
   if (chains > most) chains = most;
   const int limit = g_max_workgroups.load();
   if (limit > 0 && chains > (int64_t)limit * kWavesPerBlock) chains = (int64_t)limit * kWavesPerBlock;
@@ -1026,8 +1031,8 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
   if (err != hipSuccess) return err;
   if constexpr (!Tables::kSliced) {
     if (shadow.ordered != 0) {
-      err = launch_pos_chain<R>(stream, d, ncols, W, LB, UB, tables.A, tables.B, lrate, vexp,
-                                shadow);
+      err = launch_pos_chain<R>(stream, d, ncols, shift, W, LB, UB, tables.A, tables.B, lrate,
+                                vexp, shadow);
       if (err != hipSuccess) return err;
     }
   }
