@@ -27,12 +27,17 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE on this same command (summaries under profiles/), scaled by what the same
-# counters read for a plain copy of known size in the same run (FETCH x2.0, WRITE x1.0).
+# HBM bytes per launch of the update kernels, measured offline with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE on this same command (summaries under profiles/, named in `source`), scaled by
+# what the same counters read for a plain copy of known size in the same run (FETCH x2.0, WRITE
+# x1.0).
 HEADLINE = "sgns_v1m_d300_w5_neg5_fp32"
 MEASURED_TRAFFIC = {
     HEADLINE: {
+        # the kernels the library takes for this raw stream by itself
+        "ordered": {"neg_kernel": 29.93e9, "pos_kernel": 17.31e9,
+                    "source": "profiles/sgns_v1m_d300_ordered_step_kernel_stats_and_hbm_traffic.md"},
+        # --ordered-mode 0
         "throughput": {"neg_kernel": 29.35e9, "pos_kernel": 4.63e9,
                        "source": "profiles/sgns_v1m_d300_step_hbm_traffic.md"},
     },
@@ -471,7 +476,8 @@ def main():
     # HBM bytes per launch measured with rocprofv3 counters apply to the kernels they were taken on
     traffic = traffic_source = None
     if args.workload in MEASURED_TRAFFIC and not evaluating and not MM and args.tokens == 0 \
-            and args.wsample == 0.0 and not args.ordered_workers:
+            and args.wsample == 0.0 and not args.ordered_workers and args.rare_mode == -1 \
+            and args.max_workgroups == 0 and args.hot_mode == -1:
         key = "ordered" if args.ordered_mode != 0 else "throughput"
         m = MEASURED_TRAFFIC[args.workload].get(key)
         if m:
