@@ -109,9 +109,13 @@ hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int n
 // instance (neg_rows_available).  Launched after the throughput kernel, which returns at once
 // when the launch is ordered, as this one does when it is not.
 bool neg_rows_available(int nrows, int nwa);
+int64_t ordered_neg_chains(int waves_per_wg);   // workers, within the bound on workgroups
 hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
                            float vexp, int64_t chains, const Shadow& shadow);
+hipError_t launch_slice_neg_rows(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                 const int* WA, const int* WB, const SliceMap& m, float lrate,
+                                 float vexp, int64_t chains, const Shadow& shadow);
 // Ordered form: -1 (default) chosen per launch on the device, 0 never, 1 always.
 void set_ordered_mode(int mode);
 int get_ordered_mode();

@@ -425,6 +425,13 @@ static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int
   return hipGetLastError();
 }
 
+int64_t ordered_neg_chains(int waves_per_wg) {
+  int64_t chains = ordered_neg_workers() > 0 ? ordered_neg_workers() : kNegChains;
+  const int limit = get_max_workgroups();
+  if (limit > 0 && chains > (int64_t)limit * waves_per_wg) chains = (int64_t)limit * waves_per_wg;
+  return chains;
+}
+
 template <int R, int MAXB>
 static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, int idlimit, int nwa,
                                       int nwb, const int* WA, const int* WB, float* A, float* B,
@@ -448,9 +455,8 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   // ordered launches: the row-by-row kernel where it has an instance for the shape, else this
   // kernel on a few workgroups
   const bool rows = shadow.ordered != 0 && neg_rows_available(d, nwa);
-  int64_t chains = ordered_neg_workers() > 0 ? ordered_neg_workers() : kNegChains;
+  const int64_t chains = ordered_neg_chains(kNegWaves);
   const int limit = get_max_workgroups();
-  if (limit > 0 && chains > (int64_t)limit * kNegWaves) chains = (int64_t)limit * kNegWaves;
   int64_t per_wg_ordered = 0;
   if (shadow.ordered != 0 && !rows) {
     int64_t wgs = kNegFallbackChains / kNegWaves;

@@ -24,10 +24,12 @@ namespace w2v {
 
 namespace {
 
-template <int R, int MAXA>
+// `tables` places a word's column and, for a sliced model, says which pairs are trained and
+// which columns are written (BIDMach_CPUMACH.c:315-349 and :369-381).
+template <int R, int MAXA, class Tables>
 __global__ void __launch_bounds__(kBlock, 1)
 neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_chain,
-                const int* __restrict__ WA, const int* __restrict__ WB, float* A, float* B,
+                const int* __restrict__ WA, const int* __restrict__ WB, Tables tables,
                 float lrate, float vexp, int smode, Shadow shadow_arg) {
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
@@ -55,12 +57,18 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
     const float sbl = wb_l >= 0 ? scale_of(wb_l, vexp, smode) : 0.0f;
 
     float a[MAXA][R], daa[MAXA][R];
-    int wa[MAXA];
+    float* acol[MAXA];
+    int fa[MAXA];
 #pragma unroll
     for (int j = 0; j < MAXA; ++j) {
-      wa[j] = -1;
-      if (j < nwa) wa[j] = read_lane(wa_l, j);
-      if (wa[j] >= 0) load_col_fresh<R>(a[j], A + (int64_t)wa[j] * d, lane, d);
+      fa[j] = 0;
+      acol[j] = nullptr;
+      if (j < nwa) {
+        const ColRef ra = tables.a(read_lane(wa_l, j), d);
+        fa[j] = ra.flags;
+        acol[j] = ra.col;
+      }
+      if (fa[j] != 0) load_col_fresh<R>(a[j], acol[j], lane, d);
       zero_col<R>(daa[j]);
     }
 
@@ -72,67 +80,94 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
     const unsigned long long repeats = __ballot(seen_before && wb_l >= 0);
 
     float bn[R];
-    int wbn = read_lane(wb_l, 0);
-    if (wbn >= 0) load_col_fresh<R>(bn, B + (int64_t)wbn * d, lane, d);
+    ColRef rbn = tables.b(read_lane(wb_l, 0), d);
+    if (rbn.flags != 0) load_col_fresh<R>(bn, rbn.col, lane, d);
     for (int k = 0; k < nwb; ++k) {
-      const int wb = wbn;
+      const ColRef rb = rbn;
       float b[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) b[r] = bn[r];
       bool again = false;
       if (k + 1 < nwb) {
-        wbn = read_lane(wb_l, k + 1);
-        again = wbn >= 0 && ((repeats >> (k + 1)) & 1ull) != 0;
-        if (wbn >= 0 && !again) load_col_fresh<R>(bn, B + (int64_t)wbn * d, lane, d);
+        rbn = tables.b(read_lane(wb_l, k + 1), d);
+        again = rbn.flags != 0 && ((repeats >> (k + 1)) & 1ull) != 0;
+        if (rbn.flags != 0 && !again) load_col_fresh<R>(bn, rbn.col, lane, d);
       }
-      if (wb < 0) continue;
-      float pre = 0.0f;
+      if (rb.flags != 0) {
+        float pre = 0.0f;
 #pragma unroll
-      for (int j = 0; j < MAXA; ++j) {
-        if (wa[j] >= 0) {
-          const float s = wave_sum(dot_partial<R>(a[j], b));
-          pre = (lane == j) ? s : pre;
+        for (int j = 0; j < MAXA; ++j) {
+          if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
+            const float s = wave_sum(dot_partial<R>(a[j], b));
+            pre = (lane == j) ? s : pre;
+          }
         }
-      }
-      const float gl = -lrate * sat_sigmoid(pre);
-      const float bs = read_lane(sbl, k);
-      float dbb[R];
-      zero_col<R>(dbb);
+        const float gl = -lrate * sat_sigmoid(pre);
+        const float bs = read_lane(sbl, k);
+        float dbb[R];
+        zero_col<R>(dbb);
 #pragma unroll
-      for (int j = 0; j < MAXA; ++j) {
-        if (wa[j] >= 0) {
-          const float g = read_lane(gl, j);
-          axpy<R>(dbb, bs * g, a[j]);
-          axpy<R>(daa[j], read_lane(sal, j) * g, b);
+        for (int j = 0; j < MAXA; ++j) {
+          if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
+            const float g = read_lane(gl, j);
+            axpy<R>(dbb, bs * g, a[j]);
+            axpy<R>(daa[j], read_lane(sal, j) * g, b);
+          }
         }
+        if (tables.written(rb.flags)) atomic_add_col<R>(rb.col, dbb, lane, d);
       }
-      atomic_add_col<R>(B + (int64_t)wb * d, dbb, lane, d);
       if (again) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        load_col_fresh<R>(bn, B + (int64_t)wbn * d, lane, d);
+        load_col_fresh<R>(bn, rbn.col, lane, d);
       }
     }
 #pragma unroll
     for (int j = 0; j < MAXA; ++j)
-      if (wa[j] >= 0) atomic_add_col<R>(A + (int64_t)wa[j] * d, daa[j], lane, d);
+      if (fa[j] != 0 && tables.written(fa[j])) atomic_add_col<R>(acol[j], daa[j], lane, d);
   }
 }
 
 constexpr int64_t kMinGroupsPerChain = 16;
 
-template <int R, int MAXA>
+template <int R, int MAXA, class Tables>
 hipError_t launch_rows(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
-                       const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
+                       const int* WA, const int* WB, const Tables& tables, float lrate, float vexp,
                        int64_t chains, const Shadow& shadow) {
   const int64_t by_size = ((int64_t)ngroups + kMinGroupsPerChain - 1) / kMinGroupsPerChain;
   if (chains > by_size) chains = by_size;
   if (chains < 1) chains = 1;
   const int64_t per_chain = ((int64_t)ngroups + chains - 1) / chains;   // waves beyond: empty range
-  hipLaunchKernelGGL((neg_rows_kernel<R, MAXA>),
+  hipLaunchKernelGGL((neg_rows_kernel<R, MAXA, Tables>),
                      dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
-                     dim3(kBlock), 0, stream, d, ngroups, idlimit, nwa, nwb, per_chain, WA, WB, A,
-                     B, lrate, vexp, scale_mode(vexp), shadow);
+                     dim3(kBlock), 0, stream, d, ngroups, idlimit, nwa, nwb, per_chain, WA, WB,
+                     tables, lrate, vexp, scale_mode(vexp), shadow);
   return hipGetLastError();
+}
+
+template <class Tables>
+hipError_t launch_rows_for(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                           const int* WA, const int* WB, const Tables& tables, float lrate,
+                           float vexp, int64_t chains, const Shadow& shadow) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+  if (nwa <= 5) {
+#define CALL(R)                                                                                \
+  return launch_rows<R, 5>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp, \
+                           chains, shadow)
+    W2V_ROUNDS_SWITCH(rounds, CALL)
+#undef CALL
+  }
+  if (nwa <= 16 && rounds <= 8) {
+    switch (rounds) {
+#define CALL(R)                                                                                  \
+  case R:                                                                                        \
+    return launch_rows<R, 16>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp, \
+                              chains, shadow)
+      CALL(1); CALL(2); CALL(3); CALL(4); CALL(5); CALL(6); CALL(7); CALL(8);
+#undef CALL
+      default: break;
+    }
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace
@@ -145,26 +180,15 @@ bool neg_rows_available(int nrows, int nwa) {
 hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
                            float vexp, int64_t chains, const Shadow& shadow) {
-  const int rounds = (nrows + kWave - 1) / kWave;
-  if (nwa <= 5) {
-#define CALL(R)                                                                                \
-  return launch_rows<R, 5>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp, \
-                           chains, shadow)
-    W2V_ROUNDS_SWITCH(rounds, CALL)
-#undef CALL
-  }
-  if (nwa <= 16 && rounds <= 8) {
-    switch (rounds) {
-#define CALL(R)                                                                                 \
-  case R:                                                                                       \
-    return launch_rows<R, 16>(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp, \
-                              chains, shadow)
-      CALL(1); CALL(2); CALL(3); CALL(4); CALL(5); CALL(6); CALL(7); CALL(8);
-#undef CALL
-      default: break;
-    }
-  }
-  return hipErrorInvalidValue;
+  return launch_rows_for(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, PlainTables{A, B}, lrate,
+                         vexp, chains, shadow);
+}
+
+hipError_t launch_slice_neg_rows(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                 const int* WA, const int* WB, const SliceMap& m, float lrate,
+                                 float vexp, int64_t chains, const Shadow& shadow) {
+  return launch_rows_for(stream, nrows, ncols, 0x7fffffff, nwa, nwb, WA, WB, SlicedTables{m}, lrate,
+                         vexp, chains, shadow);
 }
 
 }  // namespace w2v

@@ -223,10 +223,12 @@ pos_eval_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ 
 // The ids of the next token and of its window (offsets -32..31) are fetched while the current
 // token is worked on.
 constexpr int kChainLook = 32;
-template <int R, int CH>
+// `tables` places a word's column and, for a sliced model, says which pairs are trained and
+// which columns are written (BIDMach_CPUMACH.c:137-157).
+template <int R, int CH, class Tables>
 __global__ void __launch_bounds__(kBlock)
 pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
-                 const int* __restrict__ LB, const int* __restrict__ UB, float* A, float* B,
+                 const int* __restrict__ LB, const int* __restrict__ UB, Tables tables,
                  float lrate, float vexp, int smode, Shadow shadow_arg) {
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
@@ -255,8 +257,9 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     const int jhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 1 - i);
     const int wnear_now = wnear;
     fetch(unit + 1);
-    if (wi < 0) continue;
-    float* const acol = A + (int64_t)wi * d;
+    const ColRef pa = tables.a(wi, d);
+    if (pa.flags == 0) continue;
+    float* const acol = pa.col;
     float a[R];
     load_col_fresh<R>(a, acol, lane, d);
     float daa[R];
@@ -273,9 +276,11 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
       int wl = -1;
       if (j >= jlo && j <= jhi && j != 0)
         wl = base == -kChainLook ? wnear_now : W[i + j];
-      const bool ok = wl >= 0;
+      const int fl = tables.b(wl, d).flags;
+      const bool ok = fl != 0 && tables.trained(pa.flags, fl);
       const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
       const unsigned long long valid = __ballot(ok);
+      const unsigned long long wmask = __ballot(ok && tables.written(fl));
       // A word that stands at several offsets of the window is updated once per offset, and the
       // reference reads it again each time (:43-46 after :60): occurrence number r of a word is
       // worked on in round r, after the adds of round r - 1 have been performed.  Pairs of
@@ -307,12 +312,12 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
             }
           }
           float b[CH][R];
-          int wb[CH];
+          float* bcol[CH];
 #pragma unroll
           for (int c = 0; c < CH; ++c) {
             if (c < n) {
-              wb[c] = read_lane(wl, src[c]);
-              load_col_fresh<R>(b[c], B + (int64_t)wb[c] * d, lane, d);
+              bcol[c] = tables.b(read_lane(wl, src[c]), d).col;
+              load_col_fresh<R>(b[c], bcol[c], lane, d);
             }
           }
           float pre = 0.0f;
@@ -330,7 +335,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
               const float g = read_lane(gl, c);
               const float bs = read_lane(sl, src[c]);
               axpy<R>(daa, ascale * g, b[c]);
-              atomic_axpy_col<R>(B + (int64_t)wb[c] * d, bs * g, a, lane, d);
+              if ((wmask >> src[c]) & 1ull) atomic_axpy_col<R>(bcol[c], bs * g, a, lane, d);
             }
           }
           touched = true;
@@ -338,7 +343,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
       }
     }
     if (touched) {
-      atomic_add_col<R>(acol, daa, lane, d);
+      if (tables.written(pa.flags)) atomic_add_col<R>(acol, daa, lane, d);
       // the adds of this token are performed before the next token's columns are read
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     }
@@ -804,7 +809,7 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   else
     shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
   shadow->combine_a = shadow->combine;
-  shadow->ordered = Tables::kSliced ? 0 : ordered_flag(forced);
+  shadow->ordered = ordered_flag(forced);
   if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
   if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
@@ -952,9 +957,9 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
 constexpr int kPosChains = 128;
 constexpr int64_t kMinTokensPerChain = 64;
 
-template <int R>
+template <int R, class Tables>
 static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shift, const int* W,
-                                   const int* LB, const int* UB, float* A, float* B, float lrate,
+                                   const int* LB, const int* UB, const Tables& tables, float lrate,
                                    float vexp, const Shadow& shadow) {
   int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
   // what is bounded is the pairs in flight: a token of a window of half-width 10 has twice the
@@ -967,9 +972,9 @@ static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shi
   if (limit > 0 && chains > (int64_t)limit * kWavesPerBlock) chains = (int64_t)limit * kWavesPerBlock;
   if (chains < 1) chains = 1;
   const int64_t per_chain = ((int64_t)ncols + chains - 1) / chains;   // waves beyond: empty range
-  hipLaunchKernelGGL((pos_chain_kernel<R, PosChunk<R>::value>),
+  hipLaunchKernelGGL((pos_chain_kernel<R, PosChunk<R>::value, Tables>),
                      dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
-                     dim3(kBlock), 0, stream, d, ncols, per_chain, W, LB, UB, A, B, lrate, vexp,
+                     dim3(kBlock), 0, stream, d, ncols, per_chain, W, LB, UB, tables, lrate, vexp,
                      scale_mode(vexp), shadow);
   return hipGetLastError();
 }
@@ -1029,12 +1034,9 @@ static hipError_t launch_pos_tile_r(hipStream_t stream, int d, int ncols, int sh
                      scale_mode(vexp), shadow);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
-  if constexpr (!Tables::kSliced) {
-    if (shadow.ordered != 0) {
-      err = launch_pos_chain<R>(stream, d, ncols, shift, W, LB, UB, tables.A, tables.B, lrate,
-                                vexp, shadow);
-      if (err != hipSuccess) return err;
-    }
+  if (shadow.ordered != 0) {
+    err = launch_pos_chain<R>(stream, d, ncols, shift, W, LB, UB, tables, lrate, vexp, shadow);
+    if (err != hipSuccess) return err;
   }
   return launch_fold(stream, fold_a, fold_b, shadow, d);
 }

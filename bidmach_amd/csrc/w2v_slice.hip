@@ -142,6 +142,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
                  Shadow shadow_arg) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const Shadow shadow = TRAIN ? resolve_hot_mode(shadow_arg) : shadow_arg;
+  if (TRAIN && launch_is_ordered(shadow_arg, shadow)) return;   // neg_rows_kernel does this launch
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;
@@ -327,6 +328,7 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   if (TRAIN) {
     err = prepare_hot_mode_sliced(stream, W, ncols, nullptr, 0, m, d, nwg, kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
+    shadow.ordered = 0;   // this kernel (no tile fits in LDS) has no ordered twin
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
                      UB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials, shadow);
@@ -350,12 +352,18 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
     err = prepare_rare_words(stream, WA, (int64_t)ngroups * nwa, WB, (int64_t)ngroups * nwb,
                              0x7fffffff, ngroups, nwg * kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
+    // ordered launches go to the row-by-row kernel where it has an instance for the shape
+    if (!neg_rows_available(d, nwa)) shadow.ordered = 0;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
                      per_wg, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials,
                      shadow);
   *nparts = nwg;
-  return hipGetLastError();
+  err = hipGetLastError();
+  if (TRAIN && err == hipSuccess && shadow.ordered != 0)
+    err = launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
+                                ordered_neg_chains(kWavesPerBlock), shadow);
+  return err;
 }
 
 template <int R, bool TRAIN>

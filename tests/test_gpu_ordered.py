@@ -151,3 +151,76 @@ def test_launches_without_frequent_words_keep_the_throughput_kernels(gpu, oracle
     oracle.word2vecPos(d, 60, skip, W2, LB, UB, Ao, Bo, 0.05, 0.0, 1)
     Ag, Bg = parity.gpu_pos(gpu, d, skip, W2, LB, UB, A2, B2, 0.05, 0.0)
     assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) > 1e-3
+
+
+# ---- sliced, multi-part models (word2vecPosSlice / word2vecNegSlice) ---------------------------
+
+from tests import test_gpu_slice as sliced   # noqa: E402
+
+
+@pytest.mark.parametrize("islice,nslices,nhead,maxcols,dohead,dual", sliced.SLICINGS)
+def test_slice_updates_forced_ordered(gpu, oracle, ordered, islice, nslices, nhead, maxcols, dohead,
+                                      dual):
+    g = gpu   # (torch, CUMACH), as the sliced tests' own fixture
+    for d, vexp in ((100, 0.0), (300, 0.5)):
+        sliced.test_pos_slice_matches_oracle(g, oracle, islice, nslices, nhead, maxcols, dohead,
+                                             dual, d, vexp)
+    for d, nwa, nwb, vexp in ((100, 5, 5, 0.0), (300, 15, 5, 0.5), (130, 3, 8, 0.5)):
+        sliced.test_neg_slice_matches_oracle(g, oracle, islice, nslices, nhead, maxcols, dohead,
+                                             dual, d, nwa, nwb, vexp)
+
+
+SMALL_SLICINGS = [  # islice, nslices, nhead, maxcols, dohead: 14 words, all of them "frequent"
+    (0, 1, 0, 1 << 20, 0),
+    (1, 2, 4, 5, 0),       # head read-only, three parts
+    (0, 2, 4, 5, 1),       # head written
+    (1, 3, 6, 4, 2),       # head-head pairs trained too
+]
+
+
+@pytest.mark.parametrize("islice,nslices,nhead,maxcols,dohead", SMALL_SLICINGS)
+def test_one_worker_reproduces_the_sequential_sliced_passes(gpu, oracle, islice, nslices, nhead,
+                                                            maxcols, dohead):
+    """The sliced operators on minibatches where every update collides with the ones before it
+    (14 words, all with ids below 16, so the default takes the ordered form; one worker's range):
+    the result is the oracle's one-thread result (BIDMach_CPUMACH.c:80-184, :267-366), with the
+    rules for which pairs are trained and which columns written; with the ordered form switched
+    off the throughput kernels land visibly elsewhere."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(100 * nslices + dohead)
+    d, V, n, skip, G, nwa, nwb = 100, 14, 60, 4, 16, 5, 5
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    W = rng.integers(0, V, n).astype(np.int32)
+    W[rng.random(n) < 0.1] = -1
+    LB, UB = corpus.window_bounds(n, skip, rng)
+    WA = np.concatenate([rng.permutation(V)[:nwa] for _ in range(G)]).astype(np.int32)
+    WB = np.concatenate([rng.permutation(V)[:nwb] for _ in range(G)]).astype(np.int32)
+
+    def run(mode):
+        host, devl = sliced.model_lists(torch, A, B, islice, nslices, nhead, maxcols, False)
+        lib.w2v_set_ordered_mode(mode)
+        try:
+            assert CUMACH.word2vecPosSlice(d, n, skip, sliced.dev(torch, W), sliced.dev(torch, LB),
+                                           sliced.dev(torch, UB), devl, 0.05, 0.5, islice, nslices,
+                                           maxcols, nhead, False, dohead) == 0
+            assert CUMACH.word2vecNegSlice(d, G, nwa, nwb, sliced.dev(torch, WA),
+                                           sliced.dev(torch, WB), devl, 0.05, 0.5, islice, nslices,
+                                           maxcols, nhead, False, dohead) == 0
+        finally:
+            lib.w2v_set_ordered_mode(-1)
+        return host, [m.cpu().numpy() for m in devl]
+
+    host, got = run(-1)
+    before = [h.copy() for h in host]
+    oracle.word2vecPosSlice(d, n, skip, W, LB, UB, host, 0.05, 0.5, 1, islice, nslices, maxcols,
+                            nhead, False, dohead)
+    oracle.word2vecNegSlice(d, G, nwa, nwb, WA, WB, host, 0.05, 0.5, 1, islice, nslices, maxcols,
+                            nhead, False, dohead)
+    assert max(np.abs(h - b).max() for h, b in zip(host, before)) > 1e-2
+    err = max(np.abs(g - h).max() for g, h in zip(got, host))
+    assert err <= 2e-5, err
+    _, loose = run(0)
+    assert max(np.abs(g - h).max() for g, h in zip(loose, host)) > 50 * err + 1e-3

@@ -91,6 +91,38 @@ def gpu_run(stream):
     return score(float(r[0]), float(r[1]), G)
 
 
+def gpu_run_sliced(stream, nparts=4):
+    """The same run through word2vecPosSlice / word2vecNegSlice on a model cut into `nparts`
+    separate allocations (one worker, no head: every word is the worker's own, so the arithmetic is
+    that of the single-table operators)."""
+    import torch
+    from bidmach_amd.cumach import CUMACH, check
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    Bh, Ah = corpus.init_tables(V, D, 42)
+    maxcols = (V + nparts - 1) // nparts
+    mm = []
+    for p in range(nparts):
+        mm += [dev(Bh[p * maxcols:(p + 1) * maxcols].copy()), dev(Ah[p * maxcols:(p + 1) * maxcols].copy())]
+    for i in range(NMB):
+        W, LB, UB, WA, WB, G = stream[i]
+        check(CUMACH.word2vecPosSlice(D, N, SKIP, dev(W), dev(LB), dev(UB), mm, lrate(i), 0.0,
+                                      0, 1, maxcols, 0, False, 1), "pos")
+        check(CUMACH.word2vecNegSlice(D, G, NNEG, NREUSE, dev(WA), dev(WB), mm, lrate(i) / NNEG,
+                                      0.0, 0, 1, maxcols, 0, False, 1), "neg")
+    A, B = torch.cat(mm[1::2]), torch.cat(mm[0::2])
+    W, LB, UB, WA, WB, G = stream[NMB]
+    ret = torch.zeros(2, dtype=torch.float64, device="cuda")
+    check(CUMACH.word2vecEvalPosF64(D, N, SKIP, dev(W), dev(LB), dev(UB), A, B, ret[0:1]), "epos")
+    check(CUMACH.word2vecEvalNegF64(D, G, NNEG, NREUSE, dev(WA), dev(WB), A, B, ret[1:2]), "eneg")
+    r = ret.cpu().numpy()
+    if not (bool(torch.isfinite(A).all()) and bool(torch.isfinite(B).all())):
+        return float("nan")
+    return score(float(r[0]), float(r[1]), G)
+
+
 def test_heldout_loss_subsampled_within_half_percent(oracle):
     stream = make_stream(1.0e-4)
     cpu_seq = cpu_run(oracle, stream, 1)
@@ -126,6 +158,11 @@ def test_heldout_loss_raw_stream_default_settings_within_the_oracles_own_band(or
     for g in gpu:
         assert np.isfinite(g)
         assert abs(g / cpu_seq - 1.0) <= band, (g, cpu_seq, band)
+    # the sliced operators take the same decision on the device
+    cut = gpu_run_sliced(stream)
+    print("raw: model cut into 4 parts, word2vecPosSlice / NegSlice, default settings: %.5f (%+.3f%%)"
+          % (cut, 100.0 * (cut / cpu_seq - 1.0)))
+    assert np.isfinite(cut) and abs(cut / cpu_seq - 1.0) <= band, (cut, cpu_seq, band)
     # for the record: the throughput kernels on the same stream (what the default avoids)
     try:
         lib.w2v_set_ordered_mode(0)
