@@ -456,31 +456,32 @@ int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int* WA, int* W
 
 // ---- bfloat16 tables ------------------------------------------------------------------------
 
-static int pos_bf16_impl(int nrows, int ncols, int* W, int* LB, int* UB, unsigned short* A,
-                         unsigned short* B, float lrate, float vexp, unsigned long long seed,
-                         bool sync) {
+static int pos_bf16_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB,
+                         unsigned short* A, unsigned short* B, float lrate, float vexp,
+                         unsigned long long seed, bool sync) {
   if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
   w2v::HotCols hot{};
   hipError_t err = side_buffers(nrows, &hot);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp,
-                                     seed, hot),
+  w2v::Shadow shadow{};   // for its hot-word counters: the launch may run in its ordered form
+  err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
+  return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate,
+                                     vexp, seed, hot, shadow),
                 sync);
 }
 
 int word2vecPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* UB, unsigned short* A,
                     unsigned short* B, float lrate, float vexp, unsigned long long seed) {
-  (void)shift;
-  return pos_bf16_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, true);
+  return pos_bf16_impl(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, seed, true);
 }
 
 int word2vecPosBf16Async(int nrows, int ncols, int shift, int* W, int* LB, int* UB,
                          unsigned short* A, unsigned short* B, float lrate, float vexp,
                          unsigned long long seed) {
-  (void)shift;
-  return pos_bf16_impl(nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, false);
+  return pos_bf16_impl(nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, seed, false);
 }
 
 static int neg_bf16_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB,
@@ -493,8 +494,11 @@ static int neg_bf16_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* W
   w2v::HotCols hot{};
   hipError_t err = side_buffers(nrows, &hot);
   if (err != hipSuccess) return (int)err;
+  w2v::Shadow shadow{};
+  err = shadow_buffers(&shadow);
+  if (err != hipSuccess) return (int)err;
   return finish(w2v::launch_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
-                                     vexp, seed, hot),
+                                     vexp, seed, hot, shadow),
                 sync);
 }
 

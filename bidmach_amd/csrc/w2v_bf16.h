@@ -89,6 +89,42 @@ __device__ __forceinline__ void load_col16(float (&x)[2 * RP], const uint16_t* c
   }
 }
 
+// The same with device-scope loads, for the ordered kernels (launch_is_ordered, w2v_device.h),
+// whose workers must see each other's, and their own, latest exchanges.
+template <int RP, bool ALIGNED>
+__device__ __forceinline__ void load_col16_fresh(float (&x)[2 * RP], const uint16_t* col, int lane,
+                                                 int d) {
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    const int e = r * 128 + 2 * lane;
+    if (ALIGNED) {
+      uint32_t v = 0;
+      if (e < d)
+        v = __hip_atomic_load(reinterpret_cast<const uint32_t*>(col + e), __ATOMIC_RELAXED,
+                              __HIP_MEMORY_SCOPE_AGENT);
+      x[2 * r] = __builtin_bit_cast(float, v << 16);
+      x[2 * r + 1] = __builtin_bit_cast(float, v & 0xFFFF0000U);
+    } else {
+      // each element out of the aligned word that holds it
+      uint32_t lo = 0, hi = 0;
+      if (e < d) {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(col + e);
+        const uint32_t w = __hip_atomic_load(reinterpret_cast<const uint32_t*>(addr & ~(uintptr_t)3),
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        lo = (addr & 2) ? (w >> 16) : (w & 0xFFFFU);
+      }
+      if (e + 1 < d) {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(col + e + 1);
+        const uint32_t w = __hip_atomic_load(reinterpret_cast<const uint32_t*>(addr & ~(uintptr_t)3),
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        hi = (addr & 2) ? (w >> 16) : (w & 0xFFFFU);
+      }
+      x[2 * r] = __builtin_bit_cast(float, lo << 16);
+      x[2 * r + 1] = __builtin_bit_cast(float, hi << 16);
+    }
+  }
+}
+
 __device__ __forceinline__ uint32_t cas_word(uint32_t* p, uint32_t expected, uint32_t desired) {
   __hip_atomic_compare_exchange_strong(p, &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
@@ -286,12 +322,20 @@ __host__ __device__ __forceinline__ uint32_t fold_slot(int table_b, int word) {
 // Launchers (enqueue only).  Tables are bf16, nrows x vocab, column-major.
 // `hot` holds zeroed side buffers of side_columns(hot.n) x side_stride(nrows) floats each (hot.n may be 0); the update
 // launchers leave them zeroed (they enqueue the narrowing kernel after the update kernel).
-hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                           const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                           uint64_t seed, HotCols hot);
+// `shadow` lends the launch the thread's hot-word counters: a launch that its device-side count
+// finds full of frequent words runs in its ordered form (launch_is_ordered, w2v_device.h).
+hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                           const int* LB, const int* UB, uint16_t* A, uint16_t* B, float lrate,
+                           float vexp, uint64_t seed, HotCols hot, Shadow shadow);
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
-                           float vexp, uint64_t seed, HotCols hot);
+                           float vexp, uint64_t seed, HotCols hot, Shadow shadow);
+// Ordered form of the negative pass (w2v_bf16_neg_rows.hip); false if the shape has no instance.
+bool neg_rows_bf16_available(int nrows, int nwa);
+hipError_t launch_neg_rows_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                                const int* WA, const int* WB, uint16_t* A, uint16_t* B,
+                                float lrate, float vexp, uint64_t seed, HotCols hot,
+                                int64_t chains, const Shadow& shadow);
 hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
                             HotCols hot);
 // The forward twins add their sum into the device double Retval[0].

@@ -21,12 +21,23 @@ namespace {
 
 constexpr int64_t kMinGroupsPerWave = 4;
 
+// A launch that the device-side count finds full of frequent words (launch_is_ordered,
+// w2v_device.h) is done by the row-by-row kernel of w2v_bf16_neg_rows.hip, and this kernel returns
+// at once (per_wave_ordered == 0); for a shape that kernel has no instance for, this one runs on
+// a few waves (ranges of per_wave_ordered groups; waves beyond the last range find it empty).
 template <int RP, bool ALIGNED, int MAXB, bool EVAL>
 __global__ void __launch_bounds__(kBlock)
-neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __restrict__ WA,
-                const int* __restrict__ WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                int smode, uint64_t seed, double floorv, double* __restrict__ Retval,
-                HotCols hot) {
+neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nwa, int nwb,
+                const int* __restrict__ WA, const int* __restrict__ WB, uint16_t* A, uint16_t* B,
+                float lrate, float vexp, int smode, uint64_t seed, double floorv,
+                double* __restrict__ Retval, HotCols hot, Shadow shadow_arg) {
+  if (!EVAL) {
+    const Shadow shadow = resolve_hot_mode(shadow_arg);
+    if (launch_is_ordered(shadow_arg, shadow)) {
+      if (per_wave_ordered == 0) return;
+      per_wave = per_wave_ordered;
+    }
+  }
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int copy = (blockIdx.x * kWavesPerBlock + wave) & (kTopCopies - 1);
@@ -155,10 +166,12 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int nwa, int nwb, const int* __r
   }
 }
 
+constexpr int kNegFallbackWaves = 32;   // workers of an ordered launch without a rows instance
+
 template <int RP, bool ALIGNED, int MAXB, bool EVAL>
 hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
                   const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
-                  double floorv, double* Retval, HotCols hot) {
+                  double floorv, double* Retval, HotCols hot, Shadow shadow) {
   auto kern = neg_bf16_kernel<RP, ALIGNED, MAXB, EVAL>;
   int64_t nwg = 0;
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
@@ -166,28 +179,50 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
   if (err != hipSuccess) return err;
   const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
   nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
-  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, nwa, nwb,
-                     WA, WB, A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval, hot);
+  bool rows = false;
+  int64_t per_wave_ordered = 0;
+  if (!EVAL) {
+    err = prepare_hot_mode(stream, WB, (int64_t)n * nwb, WA, (int64_t)n * nwa, nullptr, nullptr, d,
+                           nwg, kWavesPerBlock, &shadow);
+    if (err != hipSuccess) return err;
+    rows = shadow.ordered != 0 && neg_rows_bf16_available(d, nwa);
+    if (shadow.ordered != 0 && !rows) {
+      int64_t waves = kNegFallbackWaves;
+      const int limit = get_max_workgroups();
+      if (limit > 0 && waves > (int64_t)limit * kWavesPerBlock) waves = (int64_t)limit * kWavesPerBlock;
+      if (waves > nwg * kWavesPerBlock) waves = nwg * kWavesPerBlock;   // the grid that is launched
+      per_wave_ordered = ((int64_t)n + waves - 1) / waves;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave,
+                     per_wave_ordered, nwa, nwb, WA, WB, A, B, lrate, vexp, scale_mode(vexp), seed,
+                     floorv, Retval, hot, shadow);
   hipError_t lerr = hipGetLastError();
-  if (lerr != hipSuccess || EVAL || hot.n == 0) return lerr;
+  if (lerr != hipSuccess || EVAL) return lerr;
+  if (rows) {
+    lerr = launch_neg_rows_bf16(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, hot,
+                                ordered_neg_chains(kWavesPerBlock), shadow);
+    if (lerr != hipSuccess) return lerr;
+  }
+  if (hot.n == 0) return hipSuccess;
   return launch_fold_bf16(stream, d, A, B, seed, hot);
 }
 
 template <bool ALIGNED, bool EVAL>
 hipError_t dispatch(hipStream_t stream, int d, int n, int nwa, int nwb, const int* WA,
                     const int* WB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                    uint64_t seed, double floorv, double* Retval, HotCols hot) {
+                    uint64_t seed, double floorv, double* Retval, HotCols hot, Shadow shadow) {
   const int rp = (d + 127) / 128;
   if (nwb <= 5) {
 #define W2V_CALL(RP_)                                                                         \
   return launch<RP_, ALIGNED, 5, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
-                                       floorv, Retval, hot)
+                                       floorv, Retval, hot, shadow)
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
 #define W2V_CALL(RP_)                                                                         \
   return launch<RP_, ALIGNED, 8, EVAL>(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, \
-                                       floorv, Retval, hot)
+                                       floorv, Retval, hot, shadow)
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }
@@ -201,13 +236,13 @@ bool pair_aligned(int d, const void* A, const void* B) {
 
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
-                           float vexp, uint64_t seed, HotCols hot) {
+                           float vexp, uint64_t seed, HotCols hot, Shadow shadow) {
   if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
   if (pair_aligned(nrows, A, B))
     return dispatch<true, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
-                                 0.0, nullptr, hot);
+                                 0.0, nullptr, hot, shadow);
   return dispatch<false, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
-                                0.0, nullptr, hot);
+                                0.0, nullptr, hot, shadow);
 }
 
 hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
@@ -218,9 +253,9 @@ hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nw
   uint16_t* b = const_cast<uint16_t*>(B);
   if (pair_aligned(nrows, A, B))
     return dispatch<true, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0,
-                                floorv, Retval, HotCols{});
+                                floorv, Retval, HotCols{}, Shadow{});
   return dispatch<false, true>(stream, nrows, ncols, nwa, nwb, WA, WB, a, b, 0.0f, 0.0f, 0, floorv,
-                               Retval, HotCols{});
+                               Retval, HotCols{}, Shadow{});
 }
 
 }  // namespace w2v

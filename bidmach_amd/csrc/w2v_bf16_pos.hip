@@ -23,12 +23,23 @@ namespace {
 
 constexpr int64_t kMinTokensPerWave = 16;
 
-template <int RP, bool ALIGNED, bool EVAL>
+// ORDERED: the instance for launches that the device-side count finds full of frequent words
+// (launch_is_ordered, w2v_device.h).  A wave already walks its tokens and their windows in the
+// reference's order; what the ordered instance changes is how much is in flight and how fresh a
+// read is: a bounded number of workers (the grid), device-scope loads of the table columns (a
+// plain load may be served from this XCD's L2 as the column was before another worker's
+// exchange), and a wait for the side-buffer adds of a word before that word is read again.  Both
+// instances are launched; the one the launch is not for returns at once.
+template <int RP, bool ALIGNED, bool EVAL, bool ORDERED>
 __global__ void __launch_bounds__(kBlock)
 pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
                 const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A, uint16_t* B,
                 float lrate, float vexp, int smode, uint64_t seed, double floorv,
-                double* __restrict__ Retval, HotCols hot) {
+                double* __restrict__ Retval, HotCols hot, Shadow shadow_arg) {
+  if (!EVAL) {
+    const Shadow shadow = resolve_hot_mode(shadow_arg);
+    if (launch_is_ordered(shadow_arg, shadow) != ORDERED) return;
+  }
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int copy = (blockIdx.x * kWavesPerBlock + wave) & (kTopCopies - 1);
@@ -44,8 +55,15 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     uint16_t* acol = A + (int64_t)w * d;
     float a[2 * RP], daa[2 * RP];
     const bool ahot = !EVAL && w < hot.n;
-    load_col16<RP, ALIGNED>(a, acol, lane, d);
+    if (ORDERED)
+      load_col16_fresh<RP, ALIGNED>(a, acol, lane, d);
+    else
+      load_col16<RP, ALIGNED>(a, acol, lane, d);
     if (ahot) read_side<RP>(a, hot.sa, hot.n, w, lane, d);
+    // ordered instance: lane l remembers the l-th word of this window whose delta went to its
+    // side buffer and has not been waited for
+    int side_word = -1;
+    int nside = 0;
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
@@ -65,7 +83,17 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       return hi + 1;
     };
     auto load_b = [&](float (&x)[2 * RP], int word) {
-      load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
+      if (ORDERED) {
+        load_col16_fresh<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
+        if (word < hot.n && nside > 0 && __ballot(side_word == word) != 0ull) {
+          // this word was updated earlier in the window: its adds are performed before the read
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+          side_word = -1;
+          nside = 0;
+        }
+      } else {
+        load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
+      }
       if (!EVAL && word < hot.n) read_side<RP>(x, hot.sb, hot.n, word, lane, d);
     };
     int wb = 0;
@@ -97,9 +125,18 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
           daa[r] = fmaf(ga, b[r], daa[r]);
           db[r] = gb * a[r];
         }
-        if (bhot)
+        if (bhot) {
           write_side<RP>(hot.sb, hot.n, wb, copy, db, lane, d);
-        else
+          if (ORDERED) {
+            if (nside == kWave) {   // no lane left to remember it: wait for all of them
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+              side_word = -1;
+              nside = 0;
+            }
+            if (lane == nside) side_word = wb;
+            ++nside;
+          }
+        } else
           add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
       if (jnext <= hi && !ahead) load_b(bnext, wbnext);
@@ -113,6 +150,8 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
         write_side<RP>(hot.sa, hot.n, w, copy, daa, lane, d);
       else
         add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
+      // the adds of this token are performed before the next token's columns are read
+      if (ORDERED) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     }
   }
   if (EVAL) {
@@ -122,20 +161,36 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
 }
 
 template <int RP, bool ALIGNED, bool EVAL>
-hipError_t launch(hipStream_t stream, int d, int n, const int* W, const int* LB, const int* UB,
-                  uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed, double floorv,
-                  double* Retval, HotCols hot) {
-  auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL>;
+hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, const int* LB,
+                  const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
+                  double floorv, double* Retval, HotCols hot, Shadow shadow) {
+  auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL, false>;
   int64_t nwg = 0;
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
                                    kMinTokensPerWave * kWavesPerBlock, &nwg);
   if (err != hipSuccess) return err;
   const int64_t per_wave = ((int64_t)n + nwg * kWavesPerBlock - 1) / (nwg * kWavesPerBlock);
   nwg = ((int64_t)n + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+  if (!EVAL) {
+    err = prepare_hot_mode(stream, W, n, nullptr, 0, nullptr, nullptr, d, nwg, kWavesPerBlock,
+                           &shadow);
+    if (err != hipSuccess) return err;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, n, per_wave, W, LB, UB,
-                     A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval, hot);
+                     A, B, lrate, vexp, scale_mode(vexp), seed, floorv, Retval, hot, shadow);
   hipError_t lerr = hipGetLastError();
-  if (lerr != hipSuccess || EVAL || hot.n == 0) return lerr;
+  if (lerr != hipSuccess || EVAL) return lerr;
+  if (shadow.ordered != 0) {
+    const int64_t chains = ordered_pos_chains(n, shift);
+    const int64_t per_chain = ((int64_t)n + chains - 1) / chains;   // waves beyond: empty range
+    hipLaunchKernelGGL((pos_bf16_kernel<RP, ALIGNED, EVAL, !EVAL>),
+                       dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
+                       dim3(kBlock), 0, stream, d, n, per_chain, W, LB, UB, A, B, lrate, vexp,
+                       scale_mode(vexp), seed, floorv, Retval, hot, shadow);
+    lerr = hipGetLastError();
+    if (lerr != hipSuccess) return lerr;
+  }
+  if (hot.n == 0) return hipSuccess;
   return launch_fold_bf16(stream, d, A, B, seed, hot);
 }
 
@@ -225,20 +280,20 @@ hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t
   return hipGetLastError();
 }
 
-hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
-                           const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp,
-                           uint64_t seed, HotCols hot) {
+hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                           const int* LB, const int* UB, uint16_t* A, uint16_t* B, float lrate,
+                           float vexp, uint64_t seed, HotCols hot, Shadow shadow) {
   const int rp = (nrows + 127) / 128;
   if (pair_aligned(nrows, A, B)) {
-#define W2V_CALL(RP_)                                                                          \
-  return launch<RP_, true, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
-                                  nullptr, hot)
+#define W2V_CALL(RP_)                                                                       \
+  return launch<RP_, true, false>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, \
+                                  seed, 0.0, nullptr, hot, shadow)
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
-#define W2V_CALL(RP_)                                                                           \
-  return launch<RP_, false, false>(stream, nrows, ncols, W, LB, UB, A, B, lrate, vexp, seed, 0.0, \
-                                   nullptr, hot)
+#define W2V_CALL(RP_)                                                                        \
+  return launch<RP_, false, false>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, \
+                                   seed, 0.0, nullptr, hot, shadow)
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }
@@ -251,14 +306,14 @@ hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const 
   uint16_t* b = const_cast<uint16_t*>(B);
   if (pair_aligned(nrows, A, B)) {
 #define W2V_CALL(RP_)                                                                        \
-  return launch<RP_, true, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
-                                 Retval, HotCols{})
+  return launch<RP_, true, true>(stream, nrows, ncols, 0, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
+                                 Retval, HotCols{}, Shadow{})
     W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
   }
 #define W2V_CALL(RP_)                                                                         \
-  return launch<RP_, false, true>(stream, nrows, ncols, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
-                                  Retval, HotCols{})
+  return launch<RP_, false, true>(stream, nrows, ncols, 0, W, LB, UB, a, b, 0.0f, 0.0f, 0, floorv, \
+                                  Retval, HotCols{}, Shadow{})
   W2V_PAIR_ROUNDS_SWITCH(rp, W2V_CALL);
 #undef W2V_CALL
 }

@@ -110,6 +110,7 @@ hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int n
 // when the launch is ordered, as this one does when it is not.
 bool neg_rows_available(int nrows, int nwa);
 int64_t ordered_neg_chains(int waves_per_wg);   // workers, within the bound on workgroups
+int64_t ordered_pos_chains(int ncols, int shift);   // the same for the positive pass
 hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
                            float vexp, int64_t chains, const Shadow& shadow);

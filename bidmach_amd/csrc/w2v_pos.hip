@@ -957,10 +957,7 @@ static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* 
 constexpr int kPosChains = 128;
 constexpr int64_t kMinTokensPerChain = 64;
 
-template <int R, class Tables>
-static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shift, const int* W,
-                                   const int* LB, const int* UB, const Tables& tables, float lrate,
-                                   float vexp, const Shadow& shadow) {
+int64_t ordered_pos_chains(int ncols, int shift) {
   int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
   // what is bounded is the pairs in flight: a token of a window of half-width 10 has twice the
   // pairs of one of half-width 5, so half the workers
@@ -970,7 +967,14 @@ static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shi
   if (chains > most) chains = most;
   const int limit = g_max_workgroups.load();
   if (limit > 0 && chains > (int64_t)limit * kWavesPerBlock) chains = (int64_t)limit * kWavesPerBlock;
-  if (chains < 1) chains = 1;
+  return chains < 1 ? 1 : chains;
+}
+
+template <int R, class Tables>
+static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shift, const int* W,
+                                   const int* LB, const int* UB, const Tables& tables, float lrate,
+                                   float vexp, const Shadow& shadow) {
+  const int64_t chains = ordered_pos_chains(ncols, shift);
   const int64_t per_chain = ((int64_t)ncols + chains - 1) / chains;   // waves beyond: empty range
   hipLaunchKernelGGL((pos_chain_kernel<R, PosChunk<R>::value, Tables>),
                      dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),

@@ -123,6 +123,34 @@ def gpu_run_sliced(stream, nparts=4):
     return score(float(r[0]), float(r[1]), G)
 
 
+def gpu_run_bf16(stream):
+    """The same run on bfloat16 tables (word2vecPosBf16 / NegBf16, default settings: 1024
+    frequent words through fp32 side buffers, a fresh seed per call)."""
+    import torch
+    from bidmach_amd.cumach import CUMACH, check, f32_to_bf16
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    Bh, Ah = corpus.init_tables(V, D, 42)
+    A = torch.zeros(V * D, dtype=torch.int16, device="cuda")
+    B = torch.zeros(V * D, dtype=torch.int16, device="cuda")
+    f32_to_bf16(V * D, dev(Ah), A)
+    f32_to_bf16(V * D, dev(Bh), B)
+    for i in range(NMB):
+        W, LB, UB, WA, WB, G = stream[i]
+        check(CUMACH.word2vecPosBf16(D, N, SKIP, dev(W), dev(LB), dev(UB), A, B, lrate(i), 0.0,
+                                     2 * i), "pos16")
+        check(CUMACH.word2vecNegBf16(D, G, NNEG, NREUSE, dev(WA), dev(WB), A, B, lrate(i) / NNEG,
+                                     0.0, 2 * i + 1), "neg16")
+    W, LB, UB, WA, WB, G = stream[NMB]
+    ret = torch.zeros(2, dtype=torch.float64, device="cuda")
+    check(CUMACH.word2vecEvalPosBf16(D, N, SKIP, dev(W), dev(LB), dev(UB), A, B, ret[0:1]), "epos")
+    check(CUMACH.word2vecEvalNegBf16(D, G, NNEG, NREUSE, dev(WA), dev(WB), A, B, ret[1:2]), "eneg")
+    r = ret.cpu().numpy()
+    return score(float(r[0]), float(r[1]), G)
+
+
 def test_heldout_loss_subsampled_within_half_percent(oracle):
     stream = make_stream(1.0e-4)
     cpu_seq = cpu_run(oracle, stream, 1)
@@ -163,6 +191,18 @@ def test_heldout_loss_raw_stream_default_settings_within_the_oracles_own_band(or
     print("raw: model cut into 4 parts, word2vecPosSlice / NegSlice, default settings: %.5f (%+.3f%%)"
           % (cut, 100.0 * (cut / cpu_seq - 1.0)))
     assert np.isfinite(cut) and abs(cut / cpu_seq - 1.0) <= band, (cut, cpu_seq, band)
+    # and so do the bfloat16 operators (their stochastic rounding is noise on top)
+    half = gpu_run_bf16(stream)
+    print("raw: bfloat16 tables, word2vecPosBf16 / NegBf16, default settings: %.5f (%+.3f%%)"
+          % (half, 100.0 * (half / cpu_seq - 1.0)))
+    assert np.isfinite(half) and abs(half / cpu_seq - 1.0) <= band, (half, cpu_seq, band)
+    try:
+        lib.w2v_set_ordered_mode(0)
+        half_fast = gpu_run_bf16(stream)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+    print("raw: bfloat16 throughput kernels forced: %.5f (%+.1f%%)"
+          % (half_fast, 100.0 * (half_fast / cpu_seq - 1.0)))
     # for the record: the throughput kernels on the same stream (what the default avoids)
     try:
         lib.w2v_set_ordered_mode(0)
