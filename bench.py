@@ -644,14 +644,11 @@ def extra_legs(torch, lib, args, headline):
     if not args.no_cpu_baseline:
         configs["cfg2_forward_only_v100k_d300"]["cpu_baseline"] = cpu_eval_baseline(leg)
     leg.free()
-    # configuration 4: bfloat16 tables, vocab 3M, raw Zipf(1.1) stream (throughput kernels: the
-    # bfloat16 operators have no ordered form)
+    # configuration 4: bfloat16 tables, vocab 3M, raw Zipf(1.1) stream (ordered kernels by the
+    # device-side count, like the fp32 operators on the headline stream)
     leg = Leg(torch, "sgns_v3m_d300_w5_neg5_bf16", steps=4, warmup=1, distinct=2, lrate=args.lrate)
     r = leg.run()
     configs["cfg4_bf16_v3m_d300_zipf1.1"] = brief(leg, r, with_cpu_mbs=0 if args.no_cpu_baseline else 1)
-    configs["cfg4_bf16_v3m_d300_zipf1.1"]["note"] = (
-        "word2vecPosBf16 + word2vecNegBf16 have no ordered form: on this raw stream they run "
-        "as throughput kernels")
     leg.free()
     # configuration 5: dim 512, window 10, 15 negatives, 500k tokens
     leg = Leg(torch, "sgns_v1m_d512_w10_neg15_fp32", steps=4, warmup=1, distinct=2,

@@ -23,7 +23,7 @@ ALIAS_NAME = "libbidmachcuda-linux-x86_64.so"
 ALIAS_PATH = os.path.join(LIB_DIR, ALIAS_NAME)
 
 SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_neg_wide.hip", "w2v_neg_rows.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
-           "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_bf16_neg_rows.hip", "w2v_api.hip"]
+           "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_bf16_neg_rows.hip", "w2v_bf16_neg_rows_unaligned.hip", "w2v_api.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
@@ -31,6 +31,8 @@ HIPCC_FLAGS = [
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # an unroll pragma that the optimizer does not honour in one large instance is not an error
+    "-Wno-pass-failed",
 ]
 
 

@@ -200,6 +200,22 @@ __device__ __forceinline__ void cas_rest(uint16_t* col, const float (&delta)[2 *
   }
 }
 
+// cas_rest for a delta of the form scale * x, formed again where a word has to be repeated, so
+// that a caller with many exchanges in flight need not keep their deltas.
+template <int RP>
+__device__ __forceinline__ void cas_rest_axpy(uint16_t* col, float scale, const float (&x)[2 * RP],
+                                              int lane, int d, uint32_t key, uint32_t (&guess)[RP],
+                                              uint32_t (&found)[RP]) {
+  bool any = false;
+#pragma unroll
+  for (int r = 0; r < RP; ++r) any = any || found[r] != guess[r];
+  if (__ballot(any) == 0ull) return;   // the usual case: every word was exchanged at once
+  float delta[2 * RP];
+#pragma unroll
+  for (int r = 0; r < 2 * RP; ++r) delta[r] = scale * x[r];
+  cas_rest<RP>(col, delta, lane, d, key, guess, found);
+}
+
 template <int RP, bool ALIGNED>
 __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 * RP],
                                           const float (&delta)[2 * RP], int lane, int d,
@@ -303,6 +319,20 @@ __device__ __forceinline__ void read_side(float (&x)[2 * RP], const float* base,
   }
 }
 
+// The ordered kernels run a few hundred waves, too few for the extra copies to pay: they read and
+// write the main side column only (the end-of-call narrowing sums all copies either way).
+template <int RP>
+__device__ __forceinline__ void read_side_main(float (&x)[2 * RP], const float* base, int w,
+                                               int lane, int d) {
+  add_side_col<RP>(x, base + (int64_t)w * side_stride(d), lane, d);
+}
+
+template <int RP>
+__device__ __forceinline__ void write_side_main(float* base, int w, const float (&delta)[2 * RP],
+                                                int lane, int d) {
+  atomic_add_side_col<RP>(base + (int64_t)w * side_stride(d), delta, lane, d);
+}
+
 template <int RP>
 __device__ __forceinline__ void write_side(float* base, int hot_n, int w, int copy,
                                            const float (&delta)[2 * RP], int lane, int d) {
@@ -336,6 +366,10 @@ hipError_t launch_neg_rows_bf16(hipStream_t stream, int nrows, int ncols, int nw
                                 const int* WA, const int* WB, uint16_t* A, uint16_t* B,
                                 float lrate, float vexp, uint64_t seed, HotCols hot,
                                 int64_t chains, const Shadow& shadow);
+hipError_t launch_neg_rows_bf16_unaligned(hipStream_t stream, int nrows, int ncols, int nwa,
+                                          int nwb, const int* WA, const int* WB, uint16_t* A,
+                                          uint16_t* B, float lrate, float vexp, uint64_t seed,
+                                          HotCols hot, int64_t chains, const Shadow& shadow);
 hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
                             HotCols hot);
 // The forward twins add their sum into the device double Retval[0].

@@ -23,14 +23,9 @@ namespace {
 
 constexpr int64_t kMinTokensPerWave = 16;
 
-// ORDERED: the instance for launches that the device-side count finds full of frequent words
-// (launch_is_ordered, w2v_device.h).  A wave already walks its tokens and their windows in the
-// reference's order; what the ordered instance changes is how much is in flight and how fresh a
-// read is: a bounded number of workers (the grid), device-scope loads of the table columns (a
-// plain load may be served from this XCD's L2 as the column was before another worker's
-// exchange), and a wait for the side-buffer adds of a word before that word is read again.  Both
-// instances are launched; the one the launch is not for returns at once.
-template <int RP, bool ALIGNED, bool EVAL, bool ORDERED>
+// A launch that the device-side count finds full of frequent words is done by
+// pos_chain_bf16_kernel below, and this kernel returns at once (launch_is_ordered, w2v_device.h).
+template <int RP, bool ALIGNED, bool EVAL>
 __global__ void __launch_bounds__(kBlock)
 pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
                 const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A, uint16_t* B,
@@ -38,7 +33,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
                 double* __restrict__ Retval, HotCols hot, Shadow shadow_arg) {
   if (!EVAL) {
     const Shadow shadow = resolve_hot_mode(shadow_arg);
-    if (launch_is_ordered(shadow_arg, shadow) != ORDERED) return;
+    if (launch_is_ordered(shadow_arg, shadow)) return;
   }
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -55,15 +50,8 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     uint16_t* acol = A + (int64_t)w * d;
     float a[2 * RP], daa[2 * RP];
     const bool ahot = !EVAL && w < hot.n;
-    if (ORDERED)
-      load_col16_fresh<RP, ALIGNED>(a, acol, lane, d);
-    else
-      load_col16<RP, ALIGNED>(a, acol, lane, d);
+    load_col16<RP, ALIGNED>(a, acol, lane, d);
     if (ahot) read_side<RP>(a, hot.sa, hot.n, w, lane, d);
-    // ordered instance: lane l remembers the l-th word of this window whose delta went to its
-    // side buffer and has not been waited for
-    int side_word = -1;
-    int nside = 0;
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
     const float ascale = EVAL ? 1.0f : scale_of(w, vexp, smode);
@@ -83,17 +71,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       return hi + 1;
     };
     auto load_b = [&](float (&x)[2 * RP], int word) {
-      if (ORDERED) {
-        load_col16_fresh<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
-        if (word < hot.n && nside > 0 && __ballot(side_word == word) != 0ull) {
-          // this word was updated earlier in the window: its adds are performed before the read
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-          side_word = -1;
-          nside = 0;
-        }
-      } else {
-        load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
-      }
+      load_col16<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
       if (!EVAL && word < hot.n) read_side<RP>(x, hot.sb, hot.n, word, lane, d);
     };
     int wb = 0;
@@ -125,18 +103,9 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
           daa[r] = fmaf(ga, b[r], daa[r]);
           db[r] = gb * a[r];
         }
-        if (bhot) {
+        if (bhot)
           write_side<RP>(hot.sb, hot.n, wb, copy, db, lane, d);
-          if (ORDERED) {
-            if (nside == kWave) {   // no lane left to remember it: wait for all of them
-              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-              side_word = -1;
-              nside = 0;
-            }
-            if (lane == nside) side_word = wb;
-            ++nside;
-          }
-        } else
+        else
           add_col16<RP, ALIGNED>(bcol, b, db, lane, d, sr_key(seed, (uint32_t)i, (uint32_t)j));
       }
       if (jnext <= hi && !ahead) load_b(bnext, wbnext);
@@ -150,8 +119,6 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
         write_side<RP>(hot.sa, hot.n, w, copy, daa, lane, d);
       else
         add_col16<RP, ALIGNED>(acol, a, daa, lane, d, sr_key(seed, (uint32_t)i, 0U));
-      // the adds of this token are performed before the next token's columns are read
-      if (ORDERED) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     }
   }
   if (EVAL) {
@@ -160,11 +127,203 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
   }
 }
 
+// Ordered form of the update (launch_is_ordered, w2v_device.h): the token-by-token order of the
+// reference's CPU loop (BIDMach_CPUMACH.c:26-68) on a bounded number of workers, as
+// pos_chain_kernel (w2v_pos.hip) has it for fp32 tables.  A wave walks a contiguous range of
+// centre tokens one after the other; per token it reads the centre's A column and the window's B
+// columns with device-scope loads (table column plus the side buffer of a frequent word), writes
+// every B delta back at once - float atomics on the side buffer of a frequent word, else a
+// compare-and-swap with stochastic rounding, the exchanges of a chunk of columns in flight
+// together - and the A delta after the window, and waits for all of it before the next token's
+// reads.  A word that stands at several offsets of one window is worked on in rounds, occurrence
+// r after the writes of occurrence r - 1.  Every write uses the key of pos_bf16_kernel, so on a
+// minibatch without repeated words both kernels store the same bits.
+template <int RP>
+struct PosChunk16 {
+  // (larger chunks cost more registers than a wave has, and a spilled exchange result is waited
+  // for at once: 8 columns at dim 300 are slower than 4, 165 against 145 ms per 1M tokens)
+  static constexpr int value = RP <= 2 ? 8 : RP <= 6 ? 4 : 3;
+};
+
+template <int RP, bool ALIGNED, int CH>
+__global__ void __launch_bounds__(kBlock, 1)
+pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
+                      const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A,
+                      uint16_t* B, float lrate, float vexp, int smode, uint64_t seed, HotCols hot,
+                      Shadow shadow_arg) {
+  const Shadow shadow = resolve_hot_mode(shadow_arg);
+  if (!launch_is_ordered(shadow_arg, shadow)) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t chain = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t i_begin = chain * per_chain;
+  const int64_t i_end = min(i_begin + per_chain, (int64_t)n);
+
+  // the ids of the next token and of its window (offsets -32..31) are fetched while the current
+  // token is worked on
+  constexpr int kLook = 32;
+  int lb = 0, ub = 0, wnear = -1;
+  auto fetch = [&](int64_t t) {
+    lb = ub = 0;
+    wnear = -1;
+    if (t < i_end) {
+      lb = LB[t];
+      ub = UB[t];
+      const int64_t p = t + lane - kLook;
+      if (p >= 0 && p < n) wnear = W[p];
+    }
+  };
+  fetch(i_begin);
+  for (int64_t unit = i_begin; unit < i_end; ++unit) {
+    const int i = (int)unit;
+    const int wi = read_lane(wnear, kLook);
+    const int jlo = max(__builtin_amdgcn_readfirstlane(lb), -i);
+    const int jhi = min(__builtin_amdgcn_readfirstlane(ub), n - 1 - i);
+    const int wnear_now = wnear;
+    fetch(unit + 1);
+    if (wi < 0) continue;
+    uint16_t* const acol = A + (int64_t)wi * d;
+    float a[2 * RP], daa[2 * RP];
+    load_col16_fresh<RP, ALIGNED>(a, acol, lane, d);
+    if (wi < hot.n) read_side_main<RP>(a, hot.sa, wi, lane, d);
+#pragma unroll
+    for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
+    const float ascale = scale_of(wi, vexp, smode);
+    bool touched = false, a_written = false;
+    const uint32_t akey = sr_key(seed, (uint32_t)i, 0U);
+
+    const int base0 = min(jlo, -kLook);
+    for (int base = base0; base <= jhi; base += kWave) {
+      // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand (a
+      // window wider than 64 offsets is worked on in slabs, each after the writes of the last)
+      if (base != base0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      const int j = base + lane;
+      int wl = -1;
+      if (j >= jlo && j <= jhi && j != 0) wl = base == -kLook ? wnear_now : W[i + j];
+      const bool ok = wl >= 0;
+      const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
+      const unsigned long long valid = __ballot(ok);
+      int occ = 0;
+      {
+        unsigned long long m = valid;
+        while (m != 0ull) {
+          const int l = __builtin_ctzll(m);
+          m &= m - 1ull;
+          if (l < lane && read_lane(wl, l) == wl) ++occ;
+        }
+      }
+      for (int round = 0;; ++round) {
+        unsigned long long mask = __ballot(ok && occ == round);
+        if (mask == 0ull) break;
+        if (round > 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        while (mask != 0ull) {
+          int src[CH];
+          int nc = 0;
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (mask != 0ull) {
+              src[c] = __builtin_ctzll(mask);
+              mask &= mask - 1ull;
+              nc = c + 1;
+            } else {
+              src[c] = -1;
+            }
+          }
+          float b[CH][2 * RP];
+          float gbs[CH];
+          uint32_t guess[CH][RP], found[CH][RP];
+          int wb[CH];
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            wb[c] = -1;
+            if (c < nc) {
+              wb[c] = read_lane(wl, src[c]);
+              load_col16_fresh<RP, ALIGNED>(b[c], B + (int64_t)wb[c] * d, lane, d);
+              if (wb[c] < hot.n) read_side_main<RP>(b[c], hot.sb, wb[c], lane, d);
+            }
+          }
+          // lane c forms the sigmoid of the dot with context c: one evaluation per chunk
+          float pre = 0.0f;
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (c < nc) {
+              float part = 0.0f;
+#pragma unroll
+              for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[c][r], part);
+              const float sum = wave_sum(part);
+              pre = (lane == c) ? sum : pre;
+            }
+          }
+          const float gl = lrate * (1.0f - sat_sigmoid(pre));
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (c < nc) {
+              const float g = read_lane(gl, c);
+              const float ga = ascale * g;
+              const float gb = read_lane(sl, src[c]) * g;
+              gbs[c] = gb;
+              float db[2 * RP];
+#pragma unroll
+              for (int r = 0; r < 2 * RP; ++r) {
+                daa[r] = fmaf(ga, b[c][r], daa[r]);
+                db[r] = gb * a[r];
+              }
+              uint16_t* const bcol = B + (int64_t)wb[c] * d;
+              const uint32_t key = sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c]));
+              if (wb[c] < hot.n)
+                write_side_main<RP>(hot.sb, wb[c], db, lane, d);
+              else if (ALIGNED)
+                cas_first<RP>(bcol, b[c], db, lane, d, key, guess[c], found[c]);
+              else
+                add_col16<RP, false>(bcol, b[c], db, lane, d, key);
+            }
+          }
+          touched = true;
+          // after the token's last chunk the centre's delta is complete: its exchange joins
+          // those of the chunk's columns in flight
+          const bool last = mask == 0ull && __ballot(ok && occ == round + 1) == 0ull &&
+                            base + kWave > jhi;
+          uint32_t aguess[RP], afound[RP];
+          if (last) {
+            a_written = true;
+            if (wi < hot.n)
+              write_side_main<RP>(hot.sa, wi, daa, lane, d);
+            else if (ALIGNED)
+              cas_first<RP>(acol, a, daa, lane, d, akey, aguess, afound);
+            else
+              add_col16<RP, false>(acol, a, daa, lane, d, akey);
+          }
+          if (ALIGNED) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+              if (wb[c] >= hot.n)   // implies c < nc
+                cas_rest_axpy<RP>(B + (int64_t)wb[c] * d, gbs[c], a, lane, d,
+                                  sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c])), guess[c],
+                                  found[c]);
+            }
+            if (last && wi >= hot.n) cas_rest<RP>(acol, daa, lane, d, akey, aguess, afound);
+          }
+        }
+      }
+    }
+    if (touched) {
+      if (!a_written) {
+        if (wi < hot.n)
+          write_side_main<RP>(hot.sa, wi, daa, lane, d);
+        else
+          add_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
+      }
+      // the writes of this token are performed before the next token's columns are read
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    }
+  }
+}
+
 template <int RP, bool ALIGNED, bool EVAL>
 hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, const int* LB,
                   const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
                   double floorv, double* Retval, HotCols hot, Shadow shadow) {
-  auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL, false>;
+  auto kern = pos_bf16_kernel<RP, ALIGNED, EVAL>;
   int64_t nwg = 0;
   hipError_t err = persistent_grid(reinterpret_cast<const void*>(kern), kBlock, 0, n,
                                    kMinTokensPerWave * kWavesPerBlock, &nwg);
@@ -183,10 +342,10 @@ hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, con
   if (shadow.ordered != 0) {
     const int64_t chains = ordered_pos_chains(n, shift);
     const int64_t per_chain = ((int64_t)n + chains - 1) / chains;   // waves beyond: empty range
-    hipLaunchKernelGGL((pos_bf16_kernel<RP, ALIGNED, EVAL, !EVAL>),
+    hipLaunchKernelGGL((pos_chain_bf16_kernel<RP, ALIGNED, PosChunk16<RP>::value>),
                        dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
                        dim3(kBlock), 0, stream, d, n, per_chain, W, LB, UB, A, B, lrate, vexp,
-                       scale_mode(vexp), seed, floorv, Retval, hot, shadow);
+                       scale_mode(vexp), seed, hot, shadow);
     lerr = hipGetLastError();
     if (lerr != hipSuccess) return lerr;
   }
