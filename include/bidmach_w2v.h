@@ -203,8 +203,8 @@ int w2v_release_thread(void);
 int w2v_set_max_workgroups(int n);
 int w2v_get_max_workgroups(void);
 
-/* Ordered form of word2vecPos / word2vecNeg / word2vecNegFilt and of word2vecPosSlice /
- * word2vecNegSlice, process-wide.  The reference's CPU
+/* Ordered form of word2vecPos / word2vecNeg / word2vecNegFilt, of word2vecPosSlice /
+ * word2vecNegSlice and of word2vecPosBf16 / word2vecNegBf16, process-wide.  The reference's CPU
  * path keeps as many work units in flight as it has threads (BIDMach_CPUMACH.c:21-24, :197-201),
  * each of which reads a column just before it uses it and writes a B column back before it
  * reads the next (:57-61, :244-246).  On a raw (not subsampled) Zipf stream, where a tenth of
@@ -220,8 +220,7 @@ int w2v_get_max_workgroups(void);
  *      caller's subsampling, Word2Vec.scala:221-225) keep the throughput kernels.  A forced
  *      w2v_set_hot_update_mode also keeps them.
  *   0  never;  1  always.
- * Groups with more than 8 B words, and the bfloat16 operators, always use the throughput
- * kernels. */
+ * Groups with more than 8 B words always use the throughput kernels. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
 /* Number of wavefronts (workers) the ordered form of word2vecPos and of word2vecNeg / NegFilt

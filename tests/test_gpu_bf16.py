@@ -335,7 +335,7 @@ def test_empty_and_rejected_arguments_bf16(gpu):
 def test_heldout_loss_next_to_the_fp32_operators(hot_words, zipf):
     """Zipf(1.0) is the stream of the plumbing configuration, Zipf(1.1) that of the
     reduced-precision configuration; both behind the reference caller's default subsampling
-    (these operators have no ordered form, so a raw stream is not theirs to train on)."""
+    (the raw stream, which the ordered kernels take, is in tests/test_gpu_training.py)."""
     import torch
     from bidmach_amd.cumach import CUMACH, check, f32_to_bf16
     V, D, N, SKIP, NNEG, NREUSE, NMB, LR0 = 10000, 100, 100000, 5, 5, 5, 30, 0.025
