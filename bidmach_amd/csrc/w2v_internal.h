@@ -96,12 +96,14 @@ hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int
 
 // The same pass for groups with more than 8 B words (w2v_neg_wide.hip): the group's A columns are
 // staged in LDS, so nwa * ceil(nrows / 64) is bounded (hipErrorInvalidValue beyond, about 300).
+// `shadow` lends the launch the hot-word counters: a launch full of frequent words goes to the
+// row-by-row kernel below where that has an instance for the shape.
 hipError_t launch_neg_wide(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
-                           float vexp);
+                           float vexp, const Shadow& shadow);
 hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                                  const int* WA, const int* WB, const SliceMap& m, float lrate,
-                                 float vexp);
+                                 float vexp, const Shadow& shadow);
 
 // Ordered form of the negative pass (w2v_neg_rows.hip), for launches whose device-side count
 // finds them full of frequent words: `chains` waves walk the groups row by row in the

@@ -498,7 +498,8 @@ hipError_t launch_neg(hipStream_t stream, int nrows, int ncols, int idlimit, int
                       const int* WA, const int* WB, float* A, float* B, float lrate, float vexp,
                       Shadow shadow) {
   if (nwb > kMaxTileB)
-    return launch_neg_wide(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp);
+    return launch_neg_wide(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B, lrate, vexp,
+                           shadow);
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
 #define CALL(R)                                                                                   \

@@ -40,7 +40,9 @@ template <int R, int MAXB, typename Tables>
 __global__ void __launch_bounds__(kWave)
 neg_wide_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_wg,
                 const int* __restrict__ WA, const int* __restrict__ WB, Tables tables, float lrate,
-                float vexp, int smode) {
+                float vexp, int smode, Shadow shadow_arg) {
+  // a launch full of frequent words is done by neg_rows_kernel (launch_is_ordered, w2v_device.h)
+  if (shadow_arg.ordered != 0 && launch_is_ordered(shadow_arg, resolve_hot_mode(shadow_arg))) return;
   extern __shared__ float lds[];
   constexpr int RS = R * kWave;
   float* const a_old = lds;                          // [nwa][RS]
@@ -155,7 +157,7 @@ constexpr int64_t kWideMinGroupsPerWg = 64;
 template <int R, typename Tables>
 hipError_t launch_wide_r(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
                          const int* WA, const int* WB, const Tables& tables, float lrate,
-                         float vexp) {
+                         float vexp, Shadow shadow) {
   constexpr int MAXB = R <= 8 ? 8 : 4;
   auto kern = neg_wide_kernel<R, MAXB, Tables>;
   const size_t lds = ((size_t)2 * nwa * R * kWave + nwa) * sizeof(float);
@@ -169,21 +171,42 @@ hipError_t launch_wide_r(hipStream_t stream, int d, int ngroups, int idlimit, in
   if (err != hipSuccess) return err;
   const int64_t per_wg = ((int64_t)ngroups + nwg - 1) / nwg;
   nwg = ((int64_t)ngroups + per_wg - 1) / per_wg;
+  // Only the count of the launch's frequent words is wanted of `shadow` (this kernel uses no
+  // shadow copies): the launch is ordered or not, and the row-by-row kernel takes it if it is and
+  // has an instance for the shape.
+  if constexpr (Tables::kSliced)
+    err = prepare_hot_mode_sliced(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa,
+                                  tables.m, d, nwg, 1, &shadow);
+  else
+    err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa, nullptr,
+                           nullptr, d, nwg, 1, &shadow);
+  if (err != hipSuccess) return err;
+  if (!neg_rows_available(d, nwa)) shadow.ordered = 0;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kWave), lds, stream, d, ngroups, idlimit,
-                     nwa, nwb, per_wg, WA, WB, tables, lrate, vexp, scale_mode(vexp));
-  return hipGetLastError();
+                     nwa, nwb, per_wg, WA, WB, tables, lrate, vexp, scale_mode(vexp), shadow);
+  err = hipGetLastError();
+  if (err != hipSuccess || shadow.ordered == 0) return err;
+  if constexpr (Tables::kSliced)
+    return launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, tables.m, lrate, vexp,
+                                 ordered_neg_chains(kWavesPerBlock), shadow);
+  else
+    return launch_neg_rows(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables.A, tables.B, lrate,
+                           vexp, ordered_neg_chains(kWavesPerBlock), shadow);
 }
 
 template <typename Tables>
 hipError_t launch_wide(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
                        const int* WA, const int* WB, const Tables& tables, float lrate,
-                       float vexp) {
+                       float vexp, const Shadow& shadow) {
   const int rounds = (d + kWave - 1) / kWave;
-  if (rounds <= 2) return launch_wide_r<2>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp);
-  if (rounds <= 5) return launch_wide_r<5>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp);
-  if (rounds <= 8) return launch_wide_r<8>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp);
-  if (rounds <= 12) return launch_wide_r<12>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp);
-  if (rounds <= kMaxRounds) return launch_wide_r<kMaxRounds>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp);
+#define CALL(R) \
+  return launch_wide_r<R>(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables, lrate, vexp, shadow)
+  if (rounds <= 2) CALL(2);
+  if (rounds <= 5) CALL(5);
+  if (rounds <= 8) CALL(8);
+  if (rounds <= 12) CALL(12);
+  if (rounds <= kMaxRounds) CALL(kMaxRounds);
+#undef CALL
   return hipErrorInvalidValue;
 }
 
@@ -191,16 +214,16 @@ hipError_t launch_wide(hipStream_t stream, int d, int ngroups, int idlimit, int 
 
 hipError_t launch_neg_wide(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
-                           float vexp) {
+                           float vexp, const Shadow& shadow) {
   return launch_wide(stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, PlainTables{A, B}, lrate,
-                     vexp);
+                     vexp, shadow);
 }
 
 hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                                  const int* WA, const int* WB, const SliceMap& m, float lrate,
-                                 float vexp) {
+                                 float vexp, const Shadow& shadow) {
   return launch_wide(stream, nrows, ncols, 0x7FFFFFFF, nwa, nwb, WA, WB, SlicedTables{m}, lrate,
-                     vexp);
+                     vexp, shadow);
 }
 
 }  // namespace w2v

@@ -403,7 +403,7 @@ hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, i
                             const int* WA, const int* WB, const SliceMap& m, float lrate,
                             float vexp, Shadow shadow) {
   if (nwb > 8)
-    return launch_slice_neg_wide(stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate, vexp);
+    return launch_slice_neg_wide(stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate, vexp, shadow);
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
   hipError_t err = hipSuccess;

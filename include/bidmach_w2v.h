@@ -220,7 +220,7 @@ int w2v_get_max_workgroups(void);
  *      caller's subsampling, Word2Vec.scala:221-225) keep the throughput kernels.  A forced
  *      w2v_set_hot_update_mode also keeps them.
  *   0  never;  1  always.
- * Groups with more than 8 B words always use the throughput kernels. */
+ * The bfloat16 operators take at most 8 B words per group in either form. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
 /* Number of wavefronts (workers) the ordered form of word2vecPos and of word2vecNeg / NegFilt

@@ -41,7 +41,11 @@ def test_pos_update_forced_ordered(gpu, oracle, ordered, vexp, d, skip, ncentres
 @pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
                                          (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
                                          (40, 70, 3, 40), (300, 6, 2, 100), (640, 16, 4, 50),
-                                         (700, 6, 5, 50)])
+                                         (700, 6, 5, 50),
+                                         # more than 8 B words (the reference's GPU launcher
+                                         # runs 5 x 10, DNN127.cu:1434)
+                                         (300, 5, 10, 200), (100, 4, 21, 100), (64, 3, 64, 40),
+                                         (512, 16, 9, 40)])
 def test_neg_update_forced_ordered(gpu, oracle, ordered, vexp, d, nwa, nwb, G):
     # (40, 70, 3) and (700, 6, 5) have no row-by-row instance: the group-at-a-time kernel on a
     # few workgroups stands in
@@ -92,7 +96,8 @@ def test_one_worker_reproduces_the_sequential_positive_pass(gpu, oracle, d, skip
     assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
 
 
-@pytest.mark.parametrize("d,nwa,nwb", [(100, 5, 5), (300, 5, 5), (200, 12, 3)])
+@pytest.mark.parametrize("d,nwa,nwb", [(100, 5, 5), (300, 5, 5), (200, 12, 3), (300, 5, 10),
+                                       (100, 3, 14)])
 def test_one_worker_reproduces_the_sequential_negative_pass(gpu, oracle, d, nwa, nwb):
     """16 groups over 8 words (distinct inside a group's B words and inside its A words, as the
     group-level order of the reference matters only there): B columns change from row to row and
@@ -116,7 +121,8 @@ def test_one_worker_reproduces_the_sequential_negative_pass(gpu, oracle, d, nwa,
         At, Bt = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, 0.05, 0.5)
     finally:
         lib.w2v_set_ordered_mode(-1)
-    assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
+    if nwb <= 8:   # (the kernel for wider groups walks 16 groups on one wave, in order as well)
+        assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
 
 
 def test_a_word_twice_among_a_groups_b_words_sees_its_first_update(gpu, oracle):
