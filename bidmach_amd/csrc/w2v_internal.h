@@ -158,6 +158,10 @@ hipError_t launch_slice_neg(hipStream_t stream, int nrows, int ncols, int nwa, i
                             float vexp, Shadow shadow);
 // The tiled positive pass on a sliced model; *launched is false (and nothing was enqueued) when
 // no tile fits in LDS for this nrows / shift.
+// The ordered positive kernel on a sliced model, for the launcher of the per-centre kernel.
+hipError_t launch_slice_pos_chain(hipStream_t stream, int nrows, int ncols, int shift,
+                                  const int* W, const int* LB, const int* UB, const SliceMap& m,
+                                  float lrate, float vexp, const Shadow& shadow);
 hipError_t launch_slice_pos_tiled(hipStream_t stream, int nrows, int ncols, int shift,
                                   const int* W, const int* LB, const int* UB, const SliceMap& m,
                                   float lrate, float vexp, Shadow shadow, bool* launched);

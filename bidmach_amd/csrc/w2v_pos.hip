@@ -42,7 +42,12 @@ template <int R, int CH, bool TRAIN>
 __global__ void __launch_bounds__(kBlock)
 pos_kernel(int d, int ncols, int64_t per_xcd, const int* __restrict__ W,
            const int* __restrict__ LB, const int* __restrict__ UB, float* A, float* B, float lrate,
-           float vexp, int smode, double floorv, double* __restrict__ partials) {
+           float vexp, int smode, double floorv, double* __restrict__ partials,
+           Shadow shadow_arg) {
+  // a launch full of frequent words is done by pos_chain_kernel (launch_is_ordered)
+  if (TRAIN && shadow_arg.ordered != 0 &&
+      launch_is_ordered(shadow_arg, resolve_hot_mode(shadow_arg)))
+    return;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t unit = xcd_contiguous_block(per_xcd) * kWavesPerBlock + wave;
@@ -938,17 +943,6 @@ struct PosChunk {
   static constexpr int value = R <= 4 ? 12 : R <= 6 ? 10 : R <= 8 ? 8 : R <= 12 ? 5 : 3;
 };
 
-template <int R, bool TRAIN>
-static hipError_t launch_pos_r(hipStream_t stream, int d, int ncols, const int* W, const int* LB,
-                               const int* UB, float* A, float* B, float lrate, float vexp,
-                               double floorv, double* partials) {
-  const int64_t per_xcd = blocks_per_xcd(ncols);
-  const dim3 grid((unsigned)(per_xcd * kXcds));
-  hipLaunchKernelGGL((pos_kernel<R, PosChunk<R>::value, TRAIN>), grid, dim3(kBlock), 0, stream, d,
-                     ncols, per_xcd, W, LB, UB, A, B, lrate, vexp, scale_mode(vexp), floorv,
-                     partials);
-  return hipGetLastError();
-}
 
 // Workers of the ordered form: as many as keep the missed updates of the most frequent word near
 // what a few dozen CPU threads miss (a lockstep simulation of K workers lands 0.2 %, 0.6 %, 1.4 %,
@@ -1053,7 +1047,19 @@ static hipError_t launch_pos_plain_r(hipStream_t stream, int d, int ncols, int s
   hipError_t err = launch_pos_tile_r<R>(stream, d, ncols, shift, W, LB, UB, PlainTables{A, B}, A, B,
                                         lrate, vexp, shadow, &launched);
   if (err != hipSuccess || launched) return err;
-  return launch_pos_r<R, true>(stream, d, ncols, W, LB, UB, A, B, lrate, vexp, 0.0, nullptr);
+  // no tile fits in LDS: one wave per centre, or the ordered kernel if the launch's count of
+  // frequent words says so (no shadow copies here, only the count)
+  const int64_t per_xcd = blocks_per_xcd(ncols);
+  err = prepare_hot_mode(stream, W, ncols, nullptr, 0, nullptr, nullptr, d, per_xcd * kXcds,
+                         kWavesPerBlock, &shadow);
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL((pos_kernel<R, PosChunk<R>::value, true>), dim3((unsigned)(per_xcd * kXcds)),
+                     dim3(kBlock), 0, stream, d, ncols, per_xcd, W, LB, UB, A, B, lrate, vexp,
+                     scale_mode(vexp), 0.0, nullptr, shadow);
+  err = hipGetLastError();
+  if (err != hipSuccess || shadow.ordered == 0) return err;
+  return launch_pos_chain<R>(stream, d, ncols, shift, W, LB, UB, PlainTables{A, B}, lrate, vexp,
+                             shadow);
 }
 
 hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
@@ -1062,6 +1068,17 @@ hipError_t launch_pos(hipStream_t stream, int nrows, int ncols, int shift, const
   const int rounds = (nrows + kWave - 1) / kWave;
 #define CALL(R) \
   return launch_pos_plain_r<R>(stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp, shadow)
+  W2V_ROUNDS_SWITCH(rounds, CALL)
+#undef CALL
+}
+
+hipError_t launch_slice_pos_chain(hipStream_t stream, int nrows, int ncols, int shift,
+                                  const int* W, const int* LB, const int* UB, const SliceMap& m,
+                                  float lrate, float vexp, const Shadow& shadow) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+#define CALL(R)                                                                               \
+  return launch_pos_chain<R>(stream, nrows, ncols, shift, W, LB, UB, SlicedTables{m}, lrate, vexp, \
+                             shadow)
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
 }

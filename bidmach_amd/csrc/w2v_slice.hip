@@ -46,6 +46,7 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
                  float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
                  Shadow shadow_arg) {
   const Shadow shadow = TRAIN ? resolve_hot_mode(shadow_arg) : shadow_arg;
+  if (TRAIN && launch_is_ordered(shadow_arg, shadow)) return;   // pos_chain_kernel does this launch
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;
@@ -317,7 +318,7 @@ static hipError_t slice_grid(const void* kernel, int64_t units, int64_t* nwg, in
 }
 
 template <int R, bool TRAIN>
-static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const int* W,
+static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, int shift, const int* W,
                                      const int* LB, const int* UB, const SliceMap& m, float lrate,
                                      float vexp, double floorv, double* partials, int64_t* nparts,
                                      Shadow shadow) {
@@ -328,12 +329,14 @@ static hipError_t launch_slice_pos_r(hipStream_t stream, int d, int ncols, const
   if (TRAIN) {
     err = prepare_hot_mode_sliced(stream, W, ncols, nullptr, 0, m, d, nwg, kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
-    shadow.ordered = 0;   // this kernel (no tile fits in LDS) has no ordered twin
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ncols, per_wg, W, LB,
                      UB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials, shadow);
   *nparts = nwg;
-  return hipGetLastError();
+  err = hipGetLastError();
+  if (TRAIN && err == hipSuccess && shadow.ordered != 0)
+    err = launch_slice_pos_chain(stream, d, ncols, shift, W, LB, UB, m, lrate, vexp, shadow);
+  return err;
 }
 
 template <int R, int MAXB, bool TRAIN>
@@ -390,8 +393,8 @@ hipError_t launch_slice_pos(hipStream_t stream, int nrows, int ncols, int shift,
   const int rounds = (nrows + kWave - 1) / kWave;
   int64_t unused = 0;
 #define CALL(R)                                                                               \
-  err = launch_slice_pos_r<R, true>(stream, nrows, ncols, W, LB, UB, m, lrate, vexp, 0.0, nullptr, \
-                                    &unused, shadow);                                         \
+  err = launch_slice_pos_r<R, true>(stream, nrows, ncols, shift, W, LB, UB, m, lrate, vexp, 0.0,   \
+                                    nullptr, &unused, shadow);                                \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL
@@ -424,8 +427,8 @@ hipError_t launch_slice_eval_pos(hipStream_t stream, int nrows, int ncols, const
   hipError_t err = hipSuccess;
   int64_t nparts = 0;
 #define CALL(R)                                                                                   \
-  err = launch_slice_pos_r<R, false>(stream, nrows, ncols, W, LB, UB, m, 0.0f, 0.0f, floorv,      \
-                                     partials, &nparts, no_shadow());                                \
+  err = launch_slice_pos_r<R, false>(stream, nrows, ncols, 0, W, LB, UB, m, 0.0f, 0.0f, floorv,   \
+                                     partials, &nparts, no_shadow());                             \
   break
   W2V_ROUNDS_SWITCH(rounds, CALL)
 #undef CALL

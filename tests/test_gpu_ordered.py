@@ -32,7 +32,7 @@ def ordered():
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
 @pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (512, 10, 100),
                                              (1, 2, 50), (65, 3, 100), (1280, 5, 40),
-                                             (24, 40, 30)])
+                                             (24, 40, 30), (1000, 25, 30)])
 def test_pos_update_forced_ordered(gpu, oracle, ordered, vexp, d, skip, ncentres):
     parity.test_pos_update_matches_oracle(gpu, oracle, vexp, d, skip, ncentres)
 
@@ -171,6 +171,8 @@ def test_slice_updates_forced_ordered(gpu, oracle, ordered, islice, nslices, nhe
     for d, vexp in ((100, 0.0), (300, 0.5)):
         sliced.test_pos_slice_matches_oracle(g, oracle, islice, nslices, nhead, maxcols, dohead,
                                              dual, d, vexp)
+    sliced.test_pos_slice_matches_oracle(g, oracle, islice, nslices, nhead, maxcols, dohead, dual,
+                                         1000, 0.5, skip=25)   # a shape that fits no tile
     for d, nwa, nwb, vexp in ((100, 5, 5, 0.0), (300, 15, 5, 0.5), (130, 3, 8, 0.5)):
         sliced.test_neg_slice_matches_oracle(g, oracle, islice, nslices, nhead, maxcols, dohead,
                                              dual, d, nwa, nwb, vexp)

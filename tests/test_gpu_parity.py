@@ -182,7 +182,9 @@ def test_eval_floor_switch(gpu):
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 1.0, 0.75])
 @pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (512, 10, 100),
                                              (1, 2, 50), (65, 3, 100), (1280, 5, 40),
-                                             (24, 40, 30)])
+                                             (24, 40, 30),
+                                             # no tile of this shape fits in LDS: wave per centre
+                                             (1000, 25, 30)])
 def test_pos_update_matches_oracle(gpu, oracle, vexp, d, skip, ncentres):
     rng = np.random.default_rng(d * 7 + skip)
     V = 20000

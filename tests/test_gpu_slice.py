@@ -68,12 +68,12 @@ def assert_lists_close(devlist, hostlist, atol):
 @pytest.mark.parametrize("islice,nslices,nhead,maxcols,dohead,dual", SLICINGS)
 @pytest.mark.parametrize("d,vexp", [(100, 0.0), (300, 0.5), (65, 1.0)])
 def test_pos_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols, dohead, dual, d,
-                                  vexp):
+                                  vexp, skip=3):
     torch, CUMACH = gpu
     rng = np.random.default_rng(7 * d + islice)
-    V, skip = 2200, 3
+    V = 2200
     A, B = rand_tables(rng, V, d, 0.5 / math.sqrt(d) ** 0.5)
-    W, LB, UB = corpus.collision_free_pos(300, skip, V, rng)
+    W, LB, UB = corpus.collision_free_pos(300 if skip <= 3 else 30, skip, V, rng)
     W[rng.random(len(W)) < 0.03] = -1
     host, devl = model_lists(torch, A, B, islice, nslices, nhead, maxcols, dual)
     before = [h.copy() for h in host]
@@ -203,6 +203,15 @@ def test_colliding_minibatch_stays_close_to_sequential_oracle(gpu, oracle):
     worst = max(float(np.abs(g.cpu().numpy() - h).max()) for g, h in zip(devl, host))
     print("\nlargest update %.3e, largest GPU-oracle distance %.3e" % (moved, worst))
     assert moved > 1e-5 and worst < 0.05 * moved
+
+
+@pytest.mark.parametrize("islice,nslices,nhead,maxcols,dohead,dual", SLICINGS[1:4])
+def test_pos_slice_shape_that_fits_no_tile(gpu, oracle, islice, nslices, nhead, maxcols, dohead,
+                                           dual):
+    """dim 1000 with a window of +-25: not even 8 tokens and their halo fit in a CU's LDS, so the
+    wave-per-centre kernel runs."""
+    test_pos_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols, dohead, dual, 1000,
+                                  0.5, skip=25)
 
 
 def test_bad_slice_arguments_are_rejected(gpu):
