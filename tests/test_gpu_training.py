@@ -161,6 +161,28 @@ def test_heldout_loss_subsampled_within_half_percent(oracle):
     assert abs(gpu - cpu_seq) <= 0.005 * cpu_seq, (gpu, cpu_seq)
 
 
+def test_heldout_loss_between_the_two_regimes(oracle):
+    """A lighter subsampling (wsample = 3e-3) leaves a fifth of the kept tokens among the 16 most
+    frequent words (2.4 % are word 0): the throughput kernels already end 3.6 % below the
+    sequential run there (at wsample = 1e-3, with 11 % and 1.4 %, they are still within 0.2 %),
+    and the device-side count (ordered from 1/16 and 1/48) takes the ordered kernels for it.  The
+    default must stay within 1 % (observed -0.3 %; the oracle's 16-thread run +0.1 %)."""
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    stream = make_stream(3.0e-3)
+    cpu_seq = cpu_run(oracle, stream, 1)
+    gpu = gpu_run(stream)
+    try:
+        lib.w2v_set_ordered_mode(0)
+        fast = gpu_run(stream)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+    print("\nwsample 3e-3: held-out loss cpu(1 thread) %.5f, gpu default %+.3f%%, throughput "
+          "kernels forced %+.3f%%" % (cpu_seq, 100.0 * (gpu / cpu_seq - 1.0),
+                                     100.0 * (fast / cpu_seq - 1.0)))
+    assert abs(gpu / cpu_seq - 1.0) <= 0.01, (gpu, cpu_seq)
+
+
 def oracle_band(runs, seq):
     """Largest relative distance of the multi-threaded oracle runs from the sequential one, plus
     the half percent of the tolerance."""
