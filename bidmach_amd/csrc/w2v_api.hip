@@ -27,7 +27,7 @@ thread_local ThreadState t_state;
 std::atomic<double> g_eval_floor{1.0e-40};
 std::atomic<int> g_bf16_hot_words{1024};
 constexpr int kMaxBf16HotWords = 4096;
-constexpr int kMaxNwbBf16 = 8;   // the bfloat16 negative kernels hold every B column in registers
+constexpr int kMaxNwbBf16 = 64;   // a lane per B word, as for the fp32 tables
 
 // Per-thread, per-device fp32 side buffers for the frequent words of bf16 tables (A's then B's),
 // zeroed when allocated; the update launchers leave them zeroed.  They only grow.

@@ -46,16 +46,19 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
   if (last > n) last = n;
   double lsum = 0.0;
   for (int64_t i = first; i < last; ++i) {
+    // MAXB columns of B at a time: several trips only in the forward-only instance (an update
+    // of a group with more B words goes to the row-by-row kernel, w2v_bf16_neg_rows.h)
+    for (int kb = 0; kb < nwb; kb += MAXB) {
     float b[MAXB][2 * RP], dbb[MAXB][2 * RP];
     float bscale[MAXB];
     int wb[MAXB];
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       // an id below zero (the positive stream's mark for a dropped word) skips its pairs, as in
-      // the fp32 kernels; wb[k] < 0 also stands for k >= nwb from here on
+      // the fp32 kernels; wb[k] < 0 also stands for kb + k >= nwb from here on
       wb[k] = -1;
       bscale[k] = 0.0f;
-      if (k < nwb) wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + k]);
+      if (kb + k < nwb) wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + kb + k]);
       if (wb[k] >= 0) {
         load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d);
         if (!EVAL && wb[k] < hot.n) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
@@ -160,6 +163,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
         }
       }
     }
+    }
   }
   if (EVAL) {
     if (lane == 0 && lsum != 0.0) atomicAdd(Retval, lsum);
@@ -185,6 +189,12 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
     err = prepare_hot_mode(stream, WB, (int64_t)n * nwb, WA, (int64_t)n * nwa, nullptr, nullptr, d,
                            nwg, kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
+    if (nwb > MAXB) {
+      // this kernel holds a group's B columns in registers: wider groups go to the row-by-row
+      // kernel whatever the launch holds, on the ordered form's number of workers
+      if (!neg_rows_bf16_available(d, nwa)) return hipErrorInvalidValue;
+      shadow.ordered = 2;
+    }
     rows = shadow.ordered != 0 && neg_rows_bf16_available(d, nwa);
     if (shadow.ordered != 0 && !rows) {
       int64_t waves = kNegFallbackWaves;
@@ -237,7 +247,7 @@ bool pair_aligned(int d, const void* A, const void* B) {
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
                            float vexp, uint64_t seed, HotCols hot, Shadow shadow) {
-  if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
+  if (nwb < 1 || nwb > kWave) return hipErrorInvalidValue;
   if (pair_aligned(nrows, A, B))
     return dispatch<true, false>(stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate, vexp, seed,
                                  0.0, nullptr, hot, shadow);
@@ -248,7 +258,7 @@ hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, in
 hipError_t launch_eval_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                                 const int* WA, const int* WB, const uint16_t* A,
                                 const uint16_t* B, double floorv, double* Retval) {
-  if (nwb < 1 || nwb > 8) return hipErrorInvalidValue;
+  if (nwb < 1 || nwb > kWave) return hipErrorInvalidValue;
   uint16_t* a = const_cast<uint16_t*>(A);  // the forward instance never stores
   uint16_t* b = const_cast<uint16_t*>(B);
   if (pair_aligned(nrows, A, B))

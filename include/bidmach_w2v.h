@@ -146,7 +146,8 @@ int word2vecEvalNegAsync(int nrows, int ncols, int nwa, int nwb, int *WA, int *W
  * in flight).  With an odd nrows or a table on an odd 2-byte boundary the word that holds the
  * first or last element of a table reaches 2 bytes outside it; those bytes are written back
  * unchanged and must be addressable (they are inside any allocation the table is a view of).
- * nwb <= 8. */
+ * nwb <= w2v_max_nwb(); an update of groups with more than 8 B words needs nwa <= 5, or nwa <= 16
+ * with nrows <= 512 (hipErrorInvalidValue otherwise), and runs on a few hundred wavefronts. */
 int word2vecPosBf16(int nrows, int ncols, int shift, int *W, int *LB, int *UB, unsigned short *A,
                     unsigned short *B, float lrate, float vexp, unsigned long long seed);
 int word2vecNegBf16(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, unsigned short *A,
@@ -219,8 +220,7 @@ int w2v_get_max_workgroups(void);
  *      lowest, or at least 1/48 are id 0; launches without frequent words (after the reference
  *      caller's subsampling, Word2Vec.scala:221-225) keep the throughput kernels.  A forced
  *      w2v_set_hot_update_mode also keeps them.
- *   0  never;  1  always.
- * The bfloat16 operators take at most 8 B words per group in either form. */
+ *   0  never;  1  always. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
 /* Number of wavefronts (workers) the ordered form of word2vecPos and of word2vecNeg / NegFilt
@@ -262,8 +262,7 @@ int w2v_get_hot_update_mode(void);
 int w2v_set_rare_update_mode(int mode);
 int w2v_get_rare_update_mode(void);
 
-/* Limits of the kernels: largest nrows and largest nwb (fp32 tables; the bfloat16 operators take
- * nwb <= 8). */
+/* Limits of the kernels: largest nrows and largest nwb. */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
 

@@ -99,6 +99,8 @@ def test_eval_pos_bf16(gpu, oracle, d, V, N, skip):
     (100, 1000, 5000, 5, 5), (300, 5000, 6000, 5, 5), (512, 2000, 2000, 15, 5), (1, 10, 50, 1, 1),
     (64, 300, 500, 3, 2), (65, 300, 500, 7, 8), (1280, 200, 100, 5, 5), (50, 400, 300, 70, 4),
     (300, 500, 1000, 9, 1),
+    # more B words than a wave holds at once
+    (300, 500, 300, 5, 10), (100, 500, 200, 4, 21), (64, 300, 100, 3, 64),
 ])
 def test_eval_neg_bf16(gpu, oracle, d, V, G, nwa, nwb):
     torch, CUMACH = gpu
@@ -140,7 +142,9 @@ def test_pos_update_bf16(gpu, oracle, hot, vexp, d, skip, ncentres):
 @pytest.mark.parametrize("vexp", [0.0, 0.5, 0.75])
 @pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (512, 15, 5, 100),
                                          (1, 1, 1, 50), (65, 7, 8, 100), (1280, 5, 5, 30),
-                                         (40, 70, 3, 40), (300, 6, 2, 100), (130, 4, 6, 100)])
+                                         (40, 70, 3, 40), (300, 6, 2, 100), (130, 4, 6, 100),
+                                         # more than 8 B words: the row-by-row kernel
+                                         (300, 5, 10, 100), (100, 4, 21, 50), (512, 16, 9, 30)])
 def test_neg_update_bf16(gpu, oracle, hot, vexp, d, nwa, nwb, G):
     torch, CUMACH = gpu
     rng = np.random.default_rng(d * 5 + nwa)
@@ -315,7 +319,8 @@ def test_empty_and_rejected_arguments_bf16(gpu):
     assert CUMACH.word2vecPosBf16(0, 1, 5, i, i, i, t, t, 0.1, 0.0, 1) == 1
     assert CUMACH.word2vecPosBf16(1281, 1, 5, i, i, i, t, t, 0.1, 0.0, 1) == 1
     assert CUMACH.word2vecPosBf16(8, 1, 5, None, i, i, t, t, 0.1, 0.0, 1) == 1
-    assert CUMACH.word2vecNegBf16(8, 1, 2, 9, i, i, t, t, 0.1, 0.0, 1) == 1
+    assert CUMACH.word2vecNegBf16(8, 1, 2, 65, i, i, t, t, 0.1, 0.0, 1) == 1
+    assert CUMACH.word2vecNegBf16(8, 1, 17, 9, i, i, t, t, 0.1, 0.0, 1) == 1   # no wide instance
     from bidmach_amd.cumach import load_library
     assert load_library().w2v_set_bf16_hot_words(-1) == 1
     assert load_library().w2v_set_bf16_hot_words(4097) == 1
