@@ -131,7 +131,7 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
                                  sr_key(seed, (uint32_t)i, (uint32_t)k));
       }
       if (again) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        wait_for_own_writes();
         load_b(bn, wbn);
       }
     }
@@ -162,7 +162,7 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
       }
     }
     // the adds of this group are performed before the next group's columns are read
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    wait_for_own_writes();
   }
 }
 

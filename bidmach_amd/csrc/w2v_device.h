@@ -312,6 +312,15 @@ __device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow
          resolved.combine_a == kHotOff;
 }
 
+// Waits until this wave's outstanding memory operations, its float atomics and exchanges among
+// them, have been performed.  The ordered kernels call it between a worker's writes and the reads
+// that must see them.  All their writes are device-scope atomics, performed at the memory side, so
+// there is nothing in a cache to write back: the fence is of workgroup scope, which is the wait
+// alone (an agent-scope release adds a write-back of the XCD's L2, 6 ms per 1M-token pass).
+__device__ __forceinline__ void wait_for_own_writes() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
+
 // Whether this launch runs in its ordered form.  A launch that is full of frequent words (a raw,
 // un-subsampled Zipf stream: a tenth of all tokens are word 0) trains at the edge of stability at
 // the reference's step size, and what its result then depends on is how many updates of the

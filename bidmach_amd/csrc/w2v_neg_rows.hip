@@ -117,7 +117,7 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
         if (tables.written(rb.flags)) atomic_add_col<R>(rb.col, dbb, lane, d);
       }
       if (again) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        wait_for_own_writes();
         load_col_fresh<R>(bn, rbn.col, lane, d);
       }
     }

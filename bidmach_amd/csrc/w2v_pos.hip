@@ -276,7 +276,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     for (int base = base0; base <= jhi; base += kWave) {
       // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand.
       // (A window wider than 64 offsets is worked on in slabs, each after the adds of the last.)
-      if (base != base0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      if (base != base0) wait_for_own_writes();
       const int j = base + lane;
       int wl = -1;
       if (j >= jlo && j <= jhi && j != 0)
@@ -302,7 +302,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
       for (int round = 0;; ++round) {
         unsigned long long mask = __ballot(ok && occ == round);
         if (mask == 0ull) break;
-        if (round > 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (round > 0) wait_for_own_writes();
         while (mask != 0ull) {
           int src[CH];
           int n = 0;
@@ -350,7 +350,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     if (touched) {
       if (tables.written(pa.flags)) atomic_add_col<R>(acol, daa, lane, d);
       // the adds of this token are performed before the next token's columns are read
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      wait_for_own_writes();
     }
   }
 }
