@@ -96,17 +96,29 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
       const float ascale = (EVAL || wa < 0) ? 1.0f : scale_of(wa, vexp, smode);
+      // lane k forms the sigmoid (and, in the forward instance, the log term) of the dot with B
+      // column k: one evaluation per A column instead of one per pair
+      float pre = 0.0f;
+      bool live = false;
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
         if (wa >= 0 && wb[k] >= 0) {
           float part = 0.0f;
 #pragma unroll
           for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[k][r], part);
-          const float sg = sat_sigmoid(wave_sum(part));
-          if (EVAL) {
-            lsum += log(fmax(1.0 - (double)sg, floorv));
-          } else {
-            const float g = -lrate * sg;
+          const float sum = wave_sum(part);
+          pre = (lane == k) ? sum : pre;
+          live = (lane == k) ? true : live;
+        }
+      }
+      const float sgl = sat_sigmoid(pre);
+      if (EVAL) {
+        if (live) lsum += log(fmax(1.0 - (double)sgl, floorv));
+      } else {
+#pragma unroll
+        for (int k = 0; k < MAXB; ++k) {
+          if (wa >= 0 && wb[k] >= 0) {
+            const float g = -lrate * read_lane(sgl, k);
             const float ga = ascale * g;
             const float gb = bscale[k] * g;
 #pragma unroll
@@ -166,7 +178,9 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
     }
   }
   if (EVAL) {
-    if (lane == 0 && lsum != 0.0) atomicAdd(Retval, lsum);
+    // every lane holds the terms of its B column: one double atomic per wave
+    const double total = wave_sum_f64(lsum);
+    if (lane == 0 && total != 0.0) atomicAdd(Retval, total);
   }
 }
 
