@@ -120,3 +120,15 @@ def test_one_worker_lands_on_the_sequential_negative_pass(gpu, oracle, hot, d, n
           "(the pass moved the tables by %.0f steps)" % (d, hot, apart, moved))
     assert moved > 20.0
     assert apart <= (1.01 if hot else 3.0), apart
+
+
+def test_ordered_bf16_under_a_bound_on_workgroups(gpu, oracle, ordered, hot):
+    """w2v_set_max_workgroups bounds the ordered kernels' workers as well (one workgroup: four
+    workers, which then walk longer ranges)."""
+    ordered.w2v_set_max_workgroups(1)
+    try:
+        b16.test_pos_update_bf16(gpu, oracle, hot, 0.5, 300, 5, 300)
+        b16.test_neg_update_bf16(gpu, oracle, hot, 0.5, 300, 5, 5, 400)
+        b16.test_neg_update_bf16(gpu, oracle, hot, 0.0, 40, 70, 3, 40)   # the few-waves stand-in
+    finally:
+        ordered.w2v_set_max_workgroups(0)
