@@ -24,6 +24,20 @@ namespace w2v {
 
 namespace {
 
+// What bounds this kernel once it has a few hundred workers is the memory-side queue of the lines
+// that hold the most frequent B words' columns: every read and every add of a line takes its turn
+// (about 36 ns), and on a raw Zipf stream word 0 alone is read 0.4 M times and added to 0.4 M times
+// per 1.2 M groups.  The kHotWords most frequent columns of B therefore have kRowTwins twins each
+// (the per-XCD read copies of the throughput kernel, filled from the table before the launch,
+// serve as the memory): every writer adds its delta to the table column AND to every twin, so a
+// twin is the table column up to the order of the float adds, and a reader reads the twin its
+// worker number selects: a line then takes all the adds but only a quarter of the reads.  The
+// negative pass of a 1.2 M-group launch: 45 ms without twins however many workers, 30 ms with
+// four twins on 512 workers, 36 ms on the 384 the library uses.  (Single-table models, and
+// launches large enough for the read copies to exist; the twins are not read after the launch.)
+constexpr int kRowTwins = 4;
+static_assert((kRowTwins & (kRowTwins - 1)) == 0 && kRowTwins <= kXcds, "a power of two of the copies");
+
 // `tables` places a word's column and, for a sliced model, says which pairs are trained and
 // which columns are written (BIDMach_CPUMACH.c:315-349 and :369-381).
 template <int R, int MAXA, class Tables>
@@ -79,9 +93,18 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
       if (k < lane && read_lane(wb_l, k) == wb_l) seen_before = true;
     const unsigned long long repeats = __ballot(seen_before && wb_l >= 0);
 
+    // Twins of the most frequent B columns (see kRowTwins): a reader takes the twin its worker
+    // number selects, a writer adds to the table and to every twin.
+    const bool twins = !Tables::kSliced && shadow.pub_b != nullptr;
+    auto read_b = [&](float (&x)[R], const ColRef& r) {
+      const float* src = r.col;
+      if (twins && r.hot >= 0)
+        src = shadow.pub_b + ((int64_t)(chain & (kRowTwins - 1)) * kHotWords + r.hot) * d;
+      load_col_fresh<R>(x, src, lane, d);
+    };
     float bn[R];
     ColRef rbn = tables.b(read_lane(wb_l, 0), d);
-    if (rbn.flags != 0) load_col_fresh<R>(bn, rbn.col, lane, d);
+    if (rbn.flags != 0) read_b(bn, rbn);
     for (int k = 0; k < nwb; ++k) {
       const ColRef rb = rbn;
       float b[R];
@@ -91,7 +114,7 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
       if (k + 1 < nwb) {
         rbn = tables.b(read_lane(wb_l, k + 1), d);
         again = rbn.flags != 0 && ((repeats >> (k + 1)) & 1ull) != 0;
-        if (rbn.flags != 0 && !again) load_col_fresh<R>(bn, rbn.col, lane, d);
+        if (rbn.flags != 0 && !again) read_b(bn, rbn);
       }
       if (rb.flags != 0) {
         float pre = 0.0f;
@@ -114,11 +137,18 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
             axpy<R>(daa[j], read_lane(sal, j) * g, b);
           }
         }
-        if (tables.written(rb.flags)) atomic_add_col<R>(rb.col, dbb, lane, d);
+        if (tables.written(rb.flags)) {
+          atomic_add_col<R>(rb.col, dbb, lane, d);
+          if (twins && rb.hot >= 0) {
+#pragma unroll
+            for (int c = 0; c < kRowTwins; ++c)
+              atomic_add_col<R>(shadow.pub_b + ((int64_t)c * kHotWords + rb.hot) * d, dbb, lane, d);
+          }
+        }
       }
       if (again) {
         wait_for_own_writes();
-        load_col_fresh<R>(bn, rbn.col, lane, d);
+        read_b(bn, rbn);
       }
     }
 #pragma unroll
