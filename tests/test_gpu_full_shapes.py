@@ -96,15 +96,17 @@ def test_dim512_window10_neg15_full_shape(oracle):
         else:
             # This one does not train, on the CPU either (the loss ends far above the untrained
             # 1.386), and where it ends moves by several percent from one multi-threaded run of
-            # the oracle to the next: the band is that spread, measured here, plus 5 %.
+            # the oracle to the next (16 threads: 9.98 to 10.41 seen).  The run with fewer threads
+            # is the one nearer to the sequential order: the device is compared with an 8-thread
+            # run, within the distance of the 16-thread run from it plus 5 %.
             assert ref > 5.0
-            others = [heldout(*cpu_train(t))[0] for t in (16, 8)]
-            band = max(abs(o / ref - 1.0) for o in others) + 0.05
-            print("raw stream: the oracle again, 16 and 8 threads: %s; band %.1f%%"
-                  % (", ".join("%.5f (%+.2f%%)" % (o, 100.0 * (o / ref - 1.0)) for o in others),
-                     100.0 * band))
+            ref8 = heldout(*cpu_train(8))[0]
+            band = abs(ref / ref8 - 1.0) + 0.05
+            print("raw stream: the oracle on 8 threads %.5f (16 threads %+.2f%%, gpu %+.2f%%); "
+                  "band %.1f%%" % (ref8, 100.0 * (ref / ref8 - 1.0), 100.0 * (got / ref8 - 1.0),
+                                   100.0 * band))
             assert band <= 0.25, band
-            assert abs(got / ref - 1.0) <= band, (got, ref, band)
+            assert abs(got / ref8 - 1.0) <= band, (got, ref8, band)
 
 
 def test_bf16_vocab3m_zipf11_full_shape(oracle):
