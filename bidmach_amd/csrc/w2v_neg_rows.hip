@@ -33,8 +33,9 @@ namespace {
 // twin is the table column up to the order of the float adds, and a reader reads the twin its
 // worker number selects: a line then takes all the adds but only a quarter of the reads.  The
 // negative pass of a 1.2 M-group launch: 45 ms without twins however many workers, 30 ms with
-// four twins on 512 workers, 36 ms on the 384 the library uses.  (Single-table models, and
-// launches large enough for the read copies to exist; the twins are not read after the launch.)
+// four twins on 512 workers, 36 ms on the 384 the library uses.  (Launches large enough for the
+// read copies to exist; in a sliced model the frequent columns are the first ones of part 0; the
+// twins are not read after the launch.)
 constexpr int kRowTwins = 4;
 static_assert((kRowTwins & (kRowTwins - 1)) == 0 && kRowTwins <= kXcds, "a power of two of the copies");
 
@@ -95,7 +96,7 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
 
     // Twins of the most frequent B columns (see kRowTwins): a reader takes the twin its worker
     // number selects, a writer adds to the table and to every twin.
-    const bool twins = !Tables::kSliced && shadow.pub_b != nullptr;
+    const bool twins = shadow.pub_b != nullptr;
     auto read_b = [&](float (&x)[R], const ColRef& r) {
       const float* src = r.col;
       if (twins && r.hot >= 0)
