@@ -187,6 +187,9 @@ def parse_args():
     ap.add_argument("--ordered-workers", default="",
                     help="w2v_set_ordered_workers as POS,NEG (wavefronts of the ordered kernels; "
                          "default: the library's own numbers)")
+    ap.add_argument("--ordered-copies", default="",
+                    help="w2v_set_ordered_copies as COPIES,TWINS (delta slots of the 16 most "
+                         "frequent columns in the ordered kernels; default: the library's 4,4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")
@@ -451,6 +454,9 @@ def main():
     if args.ordered_workers:
         pw, nw = (int(x) for x in args.ordered_workers.split(","))
         check(lib.w2v_set_ordered_workers(pw, nw), "w2v_set_ordered_workers")
+    if args.ordered_copies:
+        cc, tt = (int(x) for x in args.ordered_copies.split(","))
+        check(lib.w2v_set_ordered_copies(cc, tt), "w2v_set_ordered_copies")
     if args.bf16_hot_words >= 0:
         check(lib.w2v_set_bf16_hot_words(args.bf16_hot_words), "w2v_set_bf16_hot_words")
     if args.max_workgroups > 0:

@@ -605,6 +605,13 @@ int w2v_set_ordered_workers(int pos_workers, int neg_workers) {
   return 0;
 }
 
+int w2v_set_ordered_copies(int copies, int twins) {
+  if (copies < 0 || copies > w2v::kGridMaxC || twins < 1 || copies * twins > w2v::kShadows)
+    return (int)hipErrorInvalidValue;
+  w2v::set_ordered_copies(copies, twins);
+  return 0;
+}
+
 int w2v_set_rare_update_mode(int mode) {
   w2v::set_rare_update_mode(mode);
   return 0;

@@ -225,7 +225,7 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
   if (lerr != hipSuccess || EVAL) return lerr;
   if (rows) {
     lerr = launch_neg_rows_bf16(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, hot,
-                                ordered_neg_chains(kWavesPerBlock), shadow);
+                                ordered_neg_chains(kWavesPerBlock, kNegRowWorkersBf16), shadow);
     if (lerr != hipSuccess) return lerr;
   }
   if (hot.n == 0) return hipSuccess;

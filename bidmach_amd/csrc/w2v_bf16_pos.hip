@@ -340,7 +340,7 @@ hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, con
   hipError_t lerr = hipGetLastError();
   if (lerr != hipSuccess || EVAL) return lerr;
   if (shadow.ordered != 0) {
-    const int64_t chains = ordered_pos_chains(n, shift);
+    const int64_t chains = ordered_pos_chains(n, shift, kPosChainsBf16);
     const int64_t per_chain = ((int64_t)n + chains - 1) / chains;   // waves beyond: empty range
     hipLaunchKernelGGL((pos_chain_bf16_kernel<RP, ALIGNED, PosChunk16<RP>::value>),
                        dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),

@@ -250,6 +250,10 @@ struct Shadow {
   // Ordered form of the update passes (see launch_is_ordered): 0 never, 1 when the device-side
   // count finds the launch full of frequent words, 2 always.
   int ordered;
+  // Ordered form: the frequent columns are kept as grid_c x grid_r delta slots (see
+  // load_col_ordered); grid_c == 0: read and updated in place.
+  int grid_c;
+  int grid_r;
 };
 
 constexpr int kOccurSlots = 1 << 20;
@@ -364,6 +368,68 @@ struct ColRef {
 __device__ __forceinline__ int hot_index(const ColRef& ref, int combine) {
   if (combine == kHotOff) return -1;
   return (combine == kHotCombining || ref.hot < kHotWordsExact) ? ref.hot : -1;
+}
+
+// ---- the frequent columns in the ordered kernels ------------------------------------------------
+//
+// What bounds the ordered kernels once they have a few hundred workers is the memory-side queue of
+// the few cache lines that hold the most frequent words' columns: every device-scope read and
+// every add of one line takes its turn (about 36 ns), and on a raw Zipf stream word 0 alone is
+// read 0.4 M times and added to 0.4 M times per 1M-token pass.  While an ordered launch runs, a
+// frequent column (ColRef::hot >= 0) is therefore not touched in the table at all.  Its value is
+//     table column (unchanged during the launch: plain, cacheable loads)
+//   + the sum over c < grid_c of delta slot (c, r),   for any one r < grid_r,
+// where the grid_c x grid_r slots live in the shadow buffer of the table (zero between calls).  A
+// writer adds its delta to the grid_r slots (c, 0 .. grid_r - 1) of the c its worker number
+// selects: the slots (c, r) of one c are replicas of each other up to the order of the float
+// adds.  A reader sums the grid_c slots (0 .. grid_c - 1, r) of the r its worker number selects,
+// so it sees every update made so far, and one line takes 1/grid_c of the adds and 1/grid_r of the
+// reads.  grid_fold_kernel, launched right after the ordered kernel, adds the slots (c, 0) to the
+// table and clears them all.
+constexpr int kGridMaxC = 8;
+
+__device__ __forceinline__ float* grid_slot(const Shadow& sh, int which, int c, int r, int hot,
+                                            int d) {
+  return (which ? sh.a : sh.b) + ((int64_t)(c * sh.grid_r + r) * kHotWords + hot) * d;
+}
+
+// The column `ref` of table `which` (0 = B, 1 = A) as worker `worker` of an ordered launch sees it.
+template <int R>
+__device__ __forceinline__ void load_col_ordered(float (&x)[R], const ColRef& ref,
+                                                 const Shadow& sh, int which, int64_t worker,
+                                                 int lane, int d) {
+  if (ref.hot < 0 || sh.grid_c == 0) {
+    load_col_fresh<R>(x, ref.col, lane, d);
+    return;
+  }
+  const int twin = (int)((worker / sh.grid_c) % sh.grid_r);
+  float y[kGridMaxC][R];
+#pragma unroll
+  for (int c = 0; c < kGridMaxC; ++c) {
+    if (c < sh.grid_c) load_col_fresh<R>(y[c], grid_slot(sh, which, c, twin, ref.hot, d), lane, d);
+  }
+  load_col<R>(x, ref.col, lane, d);
+#pragma unroll
+  for (int c = 0; c < kGridMaxC; ++c) {
+    if (c < sh.grid_c) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) x[r] += y[c][r];
+    }
+  }
+}
+
+// col(ref) += x by worker `worker` of an ordered launch.
+template <int R>
+__device__ __forceinline__ void add_col_ordered(const ColRef& ref, const Shadow& sh, int which,
+                                                int64_t worker, const float (&x)[R], int lane,
+                                                int d) {
+  if (ref.hot < 0 || sh.grid_c == 0) {
+    atomic_add_col<R>(ref.col, x, lane, d);
+    return;
+  }
+  const int c = (int)(worker % sh.grid_c);
+  for (int r = 0; r < sh.grid_r; ++r)
+    atomic_add_col<R>(grid_slot(sh, which, c, r, ref.hot, d), x, lane, d);
 }
 
 // The read copy of hot column `hot` of table `which` (0 = B, 1 = A) for this wave's XCD, or null.
@@ -515,6 +581,8 @@ struct PlainTables {
   }
   __device__ __forceinline__ bool trained(int, int) const { return true; }
   __device__ __forceinline__ bool written(int) const { return true; }
+  // the table whose first columns are the frequent (shadowed) ones: 0 = B, 1 = A
+  __device__ __forceinline__ float* hot_base(int which) const { return which ? A : B; }
 };
 
 // A sliced, multi-part model (jni/src/BIDMach_CPUMACH.c:80-88 of the reference).  The vocabulary
@@ -561,7 +629,38 @@ struct SlicedTables {
   __device__ __forceinline__ bool written(int f) const {
     return f == kMine || (f == kHead && m.dohead > 0);
   }
+  __device__ __forceinline__ float* hot_base(int which) const { return m.mats[which ? 1 : 0]; }
 };
+
+// After an ordered kernel: adds the delta slots (c, 0) of frequent column blockIdx.x of table
+// blockIdx.y (0 = B, 1 = A) to the table column and clears all its slots (load_col_ordered).  A
+// column no worker touched has all-zero slots and is left alone, so the vocabulary may be smaller
+// than kHotWords.  Does nothing when the launch did not run in its ordered form.
+template <class Tables>
+__global__ void __launch_bounds__(kBlock)
+grid_fold_kernel(Tables tables, Shadow shadow_arg, int d) {
+  if (shadow_arg.grid_c == 0) return;
+  const Shadow shadow = resolve_hot_mode(shadow_arg);
+  if (!launch_is_ordered(shadow_arg, shadow)) return;
+  const int w = blockIdx.x, which = blockIdx.y;
+  float* const col = tables.hot_base(which) + (int64_t)w * d;
+  for (int e = threadIdx.x; e < d; e += kBlock) {
+    float sum = 0.0f;
+    bool any = false;
+    for (int c = 0; c < shadow.grid_c; ++c) {
+      for (int r = 0; r < shadow.grid_r; ++r) {
+        float* const p = grid_slot(shadow, which, c, r, w, d) + e;
+        const float v = *p;
+        if (v != 0.0f) {
+          any = true;
+          if (r == 0) sum += v;
+          *p = 0.0f;
+        }
+      }
+    }
+    if (any) col[e] += sum;
+  }
+}
 
 // Block-level sum of one double per wave, written as one partial per block.
 __device__ __forceinline__ void block_store_partial(double wave_total, double* __restrict__ partials) {

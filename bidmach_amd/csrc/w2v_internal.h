@@ -79,6 +79,20 @@ inline Shadow no_shadow() {
 // Adds the shadow copies of the hot columns into A and B and zeroes them.
 hipError_t launch_fold(hipStream_t stream, float* A, float* B, Shadow shadow, int d);
 
+// Enqueued right after an ordered kernel: moves its delta slots into the tables (grid_fold_kernel).
+template <class Tables>
+inline hipError_t launch_grid_fold(hipStream_t stream, const Tables& tables, const Shadow& shadow,
+                                   int d) {
+  if (shadow.grid_c == 0) return hipSuccess;
+  hipLaunchKernelGGL((grid_fold_kernel<Tables>), dim3(kHotWords, 2), dim3(kBlock), 0, stream,
+                     tables, shadow, d);
+  return hipGetLastError();
+}
+// Delta slots of the frequent columns in the ordered kernels (load_col_ordered): copies x twins,
+// copies * twins <= 32, copies <= 8; copies == 0 switches them off.
+void set_ordered_copies(int copies, int twins);
+void get_ordered_copies(int* copies, int* twins);
+
 // Number of per-block partial sums an Eval launch over `units` work units writes.
 int64_t eval_partials_needed(int64_t units);
 
@@ -111,8 +125,15 @@ hipError_t launch_slice_neg_wide(hipStream_t stream, int nrows, int ncols, int n
 // instance (neg_rows_available).  Launched after the throughput kernel, which returns at once
 // when the launch is ordered, as this one does when it is not.
 bool neg_rows_available(int nrows, int nwa);
-int64_t ordered_neg_chains(int waves_per_wg);   // workers, within the bound on workgroups
-int64_t ordered_pos_chains(int ncols, int shift);   // the same for the positive pass
+// Workers of the ordered kernels: the caller's built-in number (or what w2v_set_ordered_workers
+// asks for), within the bound on workgroups.
+constexpr int kNegRowWorkers = 576;        // fp32 row-by-row kernel, one row in flight per worker
+constexpr int kNegRowWorkersBf16 = 384;    // bfloat16 row-by-row kernel, which requests a row ahead
+constexpr int kPosTeams = 192;             // fp32 positive kernel, teams of kTeamWaves waves
+constexpr int kPosChainsBf16 = 128;        // bfloat16 positive kernel, single waves
+constexpr int kTeamWaves = 4;
+int64_t ordered_neg_chains(int waves_per_wg, int builtin);
+int64_t ordered_pos_chains(int ncols, int shift, int builtin);
 hipError_t launch_neg_rows(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
                            float vexp, int64_t chains, const Shadow& shadow);

@@ -388,12 +388,8 @@ hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, 
   return hipGetLastError();
 }
 
-// Workers (waves) of the ordered form.  With the row-by-row order a lockstep simulation of 256
-// workers stays within 0.2 % of the sequential held-out loss on a raw Zipf stream (512: 0.2 %,
-// 1024: 1.1 %); on the device, configuration 1 raw ends +0.33 %, +0.09 %, -0.07 %, -0.33 %, -0.82 %
-// from the sequential oracle with 256, 320, 384, 448, 512 workers (128 positive workers each time).
-// The group-at-a-time order of this file's kernel needs 32 or fewer for 1 %.
-constexpr int kNegChains = 384;
+// Workers of the group-at-a-time kernel when a launch is ordered and the row-by-row kernel has
+// no instance for its shape: that order needs 32 or fewer for 1 % of held-out loss.
 constexpr int kNegFallbackChains = 32;
 constexpr int kMaxTileB = 8;     // B columns a wave holds in registers at once
 constexpr int kMaxNwb = kWave;   // lane k of a wave holds the group's k-th B word
@@ -427,8 +423,8 @@ static hipError_t launch_neg_eval_rb(hipStream_t stream, int d, int ngroups, int
   return hipGetLastError();
 }
 
-int64_t ordered_neg_chains(int waves_per_wg) {
-  int64_t chains = ordered_neg_workers() > 0 ? ordered_neg_workers() : kNegChains;
+int64_t ordered_neg_chains(int waves_per_wg, int builtin) {
+  int64_t chains = ordered_neg_workers() > 0 ? ordered_neg_workers() : builtin;
   const int limit = get_max_workgroups();
   if (limit > 0 && chains > (int64_t)limit * waves_per_wg) chains = (int64_t)limit * waves_per_wg;
   return chains;
@@ -457,7 +453,7 @@ static hipError_t launch_neg_train_rb(hipStream_t stream, int d, int ngroups, in
   // ordered launches: the row-by-row kernel where it has an instance for the shape, else this
   // kernel on a few workgroups
   const bool rows = shadow.ordered != 0 && neg_rows_available(d, nwa);
-  const int64_t chains = ordered_neg_chains(kNegWaves);
+  const int64_t chains = ordered_neg_chains(kNegWaves, kNegRowWorkers);
   const int limit = get_max_workgroups();
   int64_t per_wg_ordered = 0;
   if (shadow.ordered != 0 && !rows) {

@@ -10,13 +10,19 @@
 // group's last dot; here a wave keeps the group's A columns (the negatives, drawn from the
 // flatter unigram^0.75 law) and their accumulators in registers and streams the B columns through
 // one row at a time: fresh device-scope read, nwa dots, sigmoid, delta added to the table at
-// once.  The next row's column is requested while the current row is worked on.  A lockstep
-// simulation of this order stays within 0.2 % of the sequential held-out loss with 256 workers,
-// where the group-at-a-time order is 5 % off.
+// once.
 //
 // A wave is one worker and walks a contiguous range of groups, as a thread of the reference does
-// (:197-201).  Registers matter more than occupancy here (a few hundred waves run in all), so up
-// to 16 A columns stay resident.
+// (:197-201).  What the held-out loss bounds is the number of rows that are between their read and
+// their add at any time, summed over the device, and the pass runs at that number divided by the
+// time a row spends there: about 2 us for the column to arrive, then the dots, the sigmoid and the
+// add.  A row's column is therefore requested only when the row before it is done (requesting
+// it one row ahead doubles the rows in flight per worker: the same loss needs half the workers
+// and the pass takes 1.4 times as long), and the number of workers is the knob:  held-out loss of
+// the 10k-vocabulary configuration on a raw stream against the sequential oracle, 128 positive
+// workers: 384: +0.36 %, 480: +0.15 %, 576: -0.06 %, 640: -0.35 %, 768: -0.5 %.
+// Registers matter more than occupancy here (a few hundred waves run in all), so up to 16 A
+// columns stay resident.
 #include "w2v_device.h"
 #include "w2v_internal.h"
 
@@ -25,32 +31,21 @@ namespace w2v {
 namespace {
 
 // What bounds this kernel once it has a few hundred workers is the memory-side queue of the lines
-// that hold the most frequent B words' columns: every read and every add of a line takes its turn
-// (about 36 ns), and on a raw Zipf stream word 0 alone is read 0.4 M times and added to 0.4 M times
-// per 1.2 M groups.  The kHotWords most frequent columns of B therefore have kRowTwins twins each
-// (the per-XCD read copies of the throughput kernel, filled from the table before the launch,
-// serve as the memory): every writer adds its delta to the table column AND to every twin, so a
-// twin is the table column up to the order of the float adds, and a reader reads the twin its
-// worker number selects: a line then takes all the adds but only a quarter of the reads.  The
-// negative pass of a 1.2 M-group launch: 45 ms without twins however many workers, 30 ms with
-// four twins on 512 workers, 36 ms on the 384 the library uses.  (Launches large enough for the
-// read copies to exist; in a sliced model the frequent columns are the first ones of part 0; the
-// twins are not read after the launch.)
-constexpr int kRowTwins = 4;
-static_assert((kRowTwins & (kRowTwins - 1)) == 0 && kRowTwins <= kXcds, "a power of two of the copies");
-
+// that hold the most frequent B words' columns, so those columns are read and updated through the
+// delta slots of load_col_ordered / add_col_ordered (w2v_device.h): a line then takes a fraction
+// of the adds and a fraction of the reads, and no reader misses an update.  The A columns (the
+// negatives) are read and updated in place.
 // `tables` places a word's column and, for a sliced model, says which pairs are trained and
 // which columns are written (BIDMach_CPUMACH.c:315-349 and :369-381).
 template <int R, int MAXA, class Tables>
-__global__ void __launch_bounds__(kBlock, 1)
+__global__ void __launch_bounds__(kWave, 1)
 neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_chain,
                 const int* __restrict__ WA, const int* __restrict__ WB, Tables tables,
                 float lrate, float vexp, int smode, Shadow shadow_arg) {
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t chain = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int lane = threadIdx.x;
+  const int64_t chain = blockIdx.x;   // a workgroup is one wave is one worker
   const int64_t g_begin = chain * per_chain;
   const int64_t g_end = min(g_begin + per_chain, (int64_t)ngroups);
 
@@ -87,70 +82,36 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
       zero_col<R>(daa[j]);
     }
 
-    // a B word that was a B word of an earlier row of this group is read only after that row's
-    // delta has been added
-    bool seen_before = false;
-    for (int k = 0; k < nwb; ++k)
-      if (k < lane && read_lane(wb_l, k) == wb_l) seen_before = true;
-    const unsigned long long repeats = __ballot(seen_before && wb_l >= 0);
-
-    // Twins of the most frequent B columns (see kRowTwins): a reader takes the twin its worker
-    // number selects, a writer adds to the table and to every twin.
-    const bool twins = shadow.pub_b != nullptr;
-    auto read_b = [&](float (&x)[R], const ColRef& r) {
-      const float* src = r.col;
-      if (twins && r.hot >= 0)
-        src = shadow.pub_b + ((int64_t)(chain & (kRowTwins - 1)) * kHotWords + r.hot) * d;
-      load_col_fresh<R>(x, src, lane, d);
-    };
-    float bn[R];
-    ColRef rbn = tables.b(read_lane(wb_l, 0), d);
-    if (rbn.flags != 0) read_b(bn, rbn);
+    // Every row's column is read after the adds of the rows before it were issued: requests of
+    // one wave to one address are performed in order, so a B word that was a B word of an
+    // earlier row of this group is read as that row left it.
     for (int k = 0; k < nwb; ++k) {
-      const ColRef rb = rbn;
+      const ColRef rb = tables.b(read_lane(wb_l, k), d);
+      if (rb.flags == 0) continue;
       float b[R];
+      load_col_ordered<R>(b, rb, shadow, 0, chain, lane, d);
+      float pre = 0.0f;
 #pragma unroll
-      for (int r = 0; r < R; ++r) b[r] = bn[r];
-      bool again = false;
-      if (k + 1 < nwb) {
-        rbn = tables.b(read_lane(wb_l, k + 1), d);
-        again = rbn.flags != 0 && ((repeats >> (k + 1)) & 1ull) != 0;
-        if (rbn.flags != 0 && !again) read_b(bn, rbn);
-      }
-      if (rb.flags != 0) {
-        float pre = 0.0f;
-#pragma unroll
-        for (int j = 0; j < MAXA; ++j) {
-          if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
-            const float s = wave_sum(dot_partial<R>(a[j], b));
-            pre = (lane == j) ? s : pre;
-          }
-        }
-        const float gl = -lrate * sat_sigmoid(pre);
-        const float bs = read_lane(sbl, k);
-        float dbb[R];
-        zero_col<R>(dbb);
-#pragma unroll
-        for (int j = 0; j < MAXA; ++j) {
-          if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
-            const float g = read_lane(gl, j);
-            axpy<R>(dbb, bs * g, a[j]);
-            axpy<R>(daa[j], read_lane(sal, j) * g, b);
-          }
-        }
-        if (tables.written(rb.flags)) {
-          atomic_add_col<R>(rb.col, dbb, lane, d);
-          if (twins && rb.hot >= 0) {
-#pragma unroll
-            for (int c = 0; c < kRowTwins; ++c)
-              atomic_add_col<R>(shadow.pub_b + ((int64_t)c * kHotWords + rb.hot) * d, dbb, lane, d);
-          }
+      for (int j = 0; j < MAXA; ++j) {
+        if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
+          const float s = wave_sum(dot_partial<R>(a[j], b));
+          pre = (lane == j) ? s : pre;
         }
       }
-      if (again) {
-        wait_for_own_writes();
-        read_b(bn, rbn);
+      const float gl = -lrate * sat_sigmoid(pre);
+      const float bs = read_lane(sbl, k);
+      float dbb[R];
+      zero_col<R>(dbb);
+#pragma unroll
+      for (int j = 0; j < MAXA; ++j) {
+        if (fa[j] != 0 && tables.trained(fa[j], rb.flags)) {
+          const float g = read_lane(gl, j);
+          axpy<R>(dbb, bs * g, a[j]);
+          axpy<R>(daa[j], read_lane(sal, j) * g, b);
+        }
       }
+      if (tables.written(rb.flags)) add_col_ordered<R>(rb, shadow, 0, chain, dbb, lane, d);
+      wait_for_own_writes();
     }
 #pragma unroll
     for (int j = 0; j < MAXA; ++j)
@@ -168,11 +129,12 @@ hipError_t launch_rows(hipStream_t stream, int d, int ngroups, int idlimit, int 
   if (chains > by_size) chains = by_size;
   if (chains < 1) chains = 1;
   const int64_t per_chain = ((int64_t)ngroups + chains - 1) / chains;   // waves beyond: empty range
-  hipLaunchKernelGGL((neg_rows_kernel<R, MAXA, Tables>),
-                     dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
-                     dim3(kBlock), 0, stream, d, ngroups, idlimit, nwa, nwb, per_chain, WA, WB,
-                     tables, lrate, vexp, scale_mode(vexp), shadow);
-  return hipGetLastError();
+  hipLaunchKernelGGL((neg_rows_kernel<R, MAXA, Tables>), dim3((unsigned)chains), dim3(kWave), 0,
+                     stream, d, ngroups, idlimit, nwa, nwb, per_chain, WA, WB, tables, lrate, vexp,
+                     scale_mode(vexp), shadow);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return launch_grid_fold(stream, tables, shadow, d);
 }
 
 template <class Tables>

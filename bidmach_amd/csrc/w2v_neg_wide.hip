@@ -188,10 +188,10 @@ hipError_t launch_wide_r(hipStream_t stream, int d, int ngroups, int idlimit, in
   if (err != hipSuccess || shadow.ordered == 0) return err;
   if constexpr (Tables::kSliced)
     return launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, tables.m, lrate, vexp,
-                                 ordered_neg_chains(kWavesPerBlock), shadow);
+                                 ordered_neg_chains(kWavesPerBlock, kNegRowWorkers), shadow);
   else
     return launch_neg_rows(stream, d, ngroups, idlimit, nwa, nwb, WA, WB, tables.A, tables.B, lrate,
-                           vexp, ordered_neg_chains(kWavesPerBlock), shadow);
+                           vexp, ordered_neg_chains(kWavesPerBlock, kNegRowWorkers), shadow);
 }
 
 template <typename Tables>

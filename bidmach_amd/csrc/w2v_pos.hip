@@ -31,6 +31,7 @@
 // All dot products of a tile use the columns as staged (a tile is a small synchronous batch);
 // between tiles the updates are Hogwild, as between the reference's threads.
 #include <algorithm>
+#include <cstdlib>
 #include <atomic>
 
 #include "w2v_device.h"
@@ -216,30 +217,154 @@ pos_eval_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ 
 }
 
 // Ordered form of the update (launch_is_ordered, w2v_device.h): the token-by-token order of the
-// reference's CPU loop (BIDMach_CPUMACH.c:26-68).  A wave is one of a few dozen workers, like a
-// thread of the reference (:21-24): it walks a contiguous range of centre tokens one after the
-// other; for each it reads the centre's A column and the window's B columns afresh (device-scope
-// loads, so neither this CU's L1 nor this XCD's L2 can hand back a value from before another
-// worker's update), adds every B delta to the table at once and the A delta after the window,
-// and waits until those adds have been performed before it reads for the next token, whose
-// window shares all but two positions with this one.  (A tile of adjacent tokens that computes
-// from one snapshot of its columns misses exactly those updates: 16 tokens per snapshot move the
-// held-out loss of a raw Zipf stream by 5 %, 2 tokens by 1.7 %.)
+// reference's CPU loop (BIDMach_CPUMACH.c:26-68).  A worker is one of a few dozen, like a thread
+// of the reference (:21-24): it walks a contiguous range of centre tokens one after the other;
+// for each it reads the centre's A column and the window's B columns afresh (device-scope loads,
+// so neither this CU's L1 nor this XCD's L2 can hand back a value from before another worker's
+// update), adds every B delta to the table at once and the A delta after the window, and only
+// then reads for the next token, whose window shares all but two positions with this one.  (A
+// tile of adjacent tokens that computes from one snapshot of its columns misses exactly those
+// updates: 16 tokens per snapshot move the held-out loss of a raw Zipf stream by 5 %, 2 tokens
+// by 1.7 %.)
 // The ids of the next token and of its window (offsets -32..31) are fetched while the current
 // token is worked on.
+//
+// How many workers there may be is set by the held-out loss (every token in flight is a token
+// whose updates the others do not see), so what is left to make the pass faster is the time a
+// worker spends on a token: a random 1.2 KB column takes about 2 us to arrive, and a wave issues
+// the float atomics of one column in about 0.35 us.  A worker is therefore a TEAM of TW
+// wavefronts (a workgroup): the window's words are dealt to the waves by a hash of the word id,
+// each wave gathers, dots and updates the B columns of its words, the centre's column is read
+// by the wave that owns the centre's word and handed round in LDS, and the waves' shares of the
+// centre's delta meet in LDS and are added by that same wave.  A column is only ever read and
+// written by the one wave of a team that its word hashes to, so a team's accesses to one column
+// stay in program order (requests of one wave to one address are performed in order; requests of
+// different waves need not be), and one team reproduces the sequential result exactly.
 constexpr int kChainLook = 32;
+
+// The wave of a team of `tw` (a power of two) that owns word `w`.
+__device__ __forceinline__ int team_wave(int w, int tw) {
+  return (int)(((unsigned)w * 2654435761u) >> 16) & (tw - 1);
+}
+
+// One centre token worked on by one wave alone: window offsets of any reach, in slabs of 64.
+// `wnear` holds the word ids at offsets -32..31 of token i (lane l: offset l - 32).
 // `tables` places a word's column and, for a sliced model, says which pairs are trained and
 // which columns are written (BIDMach_CPUMACH.c:137-157).
 template <int R, int CH, class Tables>
-__global__ void __launch_bounds__(kBlock)
+__device__ __forceinline__ void chain_token_solo(int i, int wi, int jlo, int jhi, int wnear,
+                                                 const ColRef& pa, int d, int ncols,
+                                                 const int* __restrict__ W, const Tables& tables,
+                                                 float lrate, float vexp, int smode,
+                                                 const Shadow& shadow, int64_t chain, int lane) {
+  float a[R];
+  load_col_ordered<R>(a, pa, shadow, 1, chain, lane, d);
+  float daa[R];
+  zero_col<R>(daa);
+  const float ascale = scale_of(wi, vexp, smode);
+  bool touched = false;
+
+  const int base0 = min(jlo, -kChainLook);
+  for (int base = base0; base <= jhi; base += kWave) {
+    // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand.
+    // (A window wider than 64 offsets is worked on in slabs, each after the adds of the last.)
+    if (base != base0) wait_for_own_writes();
+    const int j = base + lane;
+    int wl = -1;
+    if (j >= jlo && j <= jhi && j != 0) wl = base == -kChainLook ? wnear : W[i + j];
+    const int fl = tables.b(wl, d).flags;
+    const bool ok = fl != 0 && tables.trained(pa.flags, fl);
+    const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
+    const unsigned long long valid = __ballot(ok);
+    const unsigned long long wmask = __ballot(ok && tables.written(fl));
+    // A word that stands at several offsets of the window is updated once per offset, and the
+    // reference reads it again each time (:43-46 after :60): occurrence number r of a word is
+    // worked on in round r, after the adds of round r - 1.  Pairs of different words commute, so
+    // the rounds change nothing else.
+    int occ = 0;
+    {
+      unsigned long long m = valid;
+      while (m != 0ull) {
+        const int l = __builtin_ctzll(m);
+        m &= m - 1ull;
+        if (l < lane && read_lane(wl, l) == wl) ++occ;
+      }
+    }
+    for (int round = 0;; ++round) {
+      unsigned long long mask = __ballot(ok && occ == round);
+      if (mask == 0ull) break;
+      if (round > 0) wait_for_own_writes();
+      while (mask != 0ull) {
+        int src[CH];
+        int n = 0;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (mask != 0ull) {
+            src[c] = __builtin_ctzll(mask);
+            mask &= mask - 1ull;
+            n = c + 1;
+          } else {
+            src[c] = -1;
+          }
+        }
+        float b[CH][R];
+        ColRef rb[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (c < n) {
+            rb[c] = tables.b(read_lane(wl, src[c]), d);
+            load_col_ordered<R>(b[c], rb[c], shadow, 0, chain, lane, d);
+          }
+        }
+        float pre = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (c < n) {
+            const float s = wave_sum(dot_partial<R>(a, b[c]));
+            pre = (lane == c) ? s : pre;
+          }
+        }
+        const float gl = lrate * (1.0f - sat_sigmoid(pre));
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          if (c < n) {
+            const float g = read_lane(gl, c);
+            const float bs = read_lane(sl, src[c]);
+            axpy<R>(daa, ascale * g, b[c]);
+            if ((wmask >> src[c]) & 1ull) {
+              float db[R];
+#pragma unroll
+              for (int r = 0; r < R; ++r) db[r] = (bs * g) * a[r];
+              add_col_ordered<R>(rb[c], shadow, 0, chain, db, lane, d);
+            }
+          }
+        }
+        touched = true;
+      }
+    }
+  }
+  if (touched && tables.written(pa.flags)) add_col_ordered<R>(pa, shadow, 1, chain, daa, lane, d);
+}
+
+// Columns a wave of a team gathers at a time: a team's wave meets a fraction of the window.
+template <int R>
+struct TeamChunk {
+  static constexpr int value = R <= 8 ? 6 : R <= 12 ? 4 : 3;
+};
+
+template <int R, int CH, int TW, class Tables>
+__global__ void __launch_bounds__(TW * kWave)
 pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
                  const int* __restrict__ LB, const int* __restrict__ UB, Tables tables,
                  float lrate, float vexp, int smode, Shadow shadow_arg) {
+  // the centre's column as its owner read it, and each wave's share of the centre's delta
+  __shared__ float s_a[TW > 1 ? R * kWave : 1];
+  __shared__ float s_da[TW > 1 ? TW : 1][TW > 1 ? R * kWave : 1];
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t chain = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t chain = blockIdx.x;   // a workgroup is a worker
   const int64_t i_begin = chain * per_chain;
   const int64_t i_end = min(i_begin + per_chain, (int64_t)ncols);
 
@@ -264,93 +389,151 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     fetch(unit + 1);
     const ColRef pa = tables.a(wi, d);
     if (pa.flags == 0) continue;
-    float* const acol = pa.col;
-    float a[R];
-    load_col_fresh<R>(a, acol, lane, d);
-    float daa[R];
-    zero_col<R>(daa);
-    const float ascale = scale_of(wi, vexp, smode);
-    bool touched = false;
-
-    const int base0 = min(jlo, -kChainLook);
-    for (int base = base0; base <= jhi; base += kWave) {
-      // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand.
-      // (A window wider than 64 offsets is worked on in slabs, each after the adds of the last.)
-      if (base != base0) wait_for_own_writes();
-      const int j = base + lane;
-      int wl = -1;
-      if (j >= jlo && j <= jhi && j != 0)
-        wl = base == -kChainLook ? wnear_now : W[i + j];
-      const int fl = tables.b(wl, d).flags;
-      const bool ok = fl != 0 && tables.trained(pa.flags, fl);
-      const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
-      const unsigned long long valid = __ballot(ok);
-      const unsigned long long wmask = __ballot(ok && tables.written(fl));
-      // A word that stands at several offsets of the window is updated once per offset, and the
-      // reference reads it again each time (:43-46 after :60): occurrence number r of a word is
-      // worked on in round r, after the adds of round r - 1 have been performed.  Pairs of
-      // different words commute, so the rounds change nothing else.
-      int occ = 0;
-      {
-        unsigned long long m = valid;
-        while (m != 0ull) {
-          const int l = __builtin_ctzll(m);
-          m &= m - 1ull;
-          if (l < lane && read_lane(wl, l) == wl) ++occ;
-        }
+    if (TW == 1) {
+      chain_token_solo<R, CH, Tables>(i, wi, jlo, jhi, wnear_now, pa, d, ncols, W, tables, lrate,
+                                      vexp, smode, shadow, chain, lane);
+      continue;
+    }
+    const int oa = team_wave(wi, TW);
+    if (jlo < -kChainLook || jhi >= kChainLook) {
+      // a window beyond the offsets a wave's lanes cover: the centre's owner does the token alone
+      // and waits for its adds to be performed before the team goes on (the next tokens read the
+      // same columns from other waves)
+      if (wave == oa) {
+        chain_token_solo<R, CH, Tables>(i, wi, jlo, jhi, wnear_now, pa, d, ncols, W, tables, lrate,
+                                        vexp, smode, shadow, chain, lane);
+        __builtin_amdgcn_s_waitcnt(0);
       }
-      for (int round = 0;; ++round) {
-        unsigned long long mask = __ballot(ok && occ == round);
-        if (mask == 0ull) break;
-        if (round > 0) wait_for_own_writes();
-        while (mask != 0ull) {
-          int src[CH];
-          int n = 0;
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (mask != 0ull) {
-              src[c] = __builtin_ctzll(mask);
-              mask &= mask - 1ull;
-              n = c + 1;
-            } else {
-              src[c] = -1;
-            }
-          }
-          float b[CH][R];
-          float* bcol[CH];
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (c < n) {
-              bcol[c] = tables.b(read_lane(wl, src[c]), d).col;
-              load_col_fresh<R>(b[c], bcol[c], lane, d);
-            }
-          }
-          float pre = 0.0f;
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (c < n) {
-              const float s = wave_sum(dot_partial<R>(a, b[c]));
-              pre = (lane == c) ? s : pre;
-            }
-          }
-          const float gl = lrate * (1.0f - sat_sigmoid(pre));
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (c < n) {
-              const float g = read_lane(gl, c);
-              const float bs = read_lane(sl, src[c]);
-              axpy<R>(daa, ascale * g, b[c]);
-              if ((wmask >> src[c]) & 1ull) atomic_axpy_col<R>(bcol[c], bs * g, a, lane, d);
-            }
-          }
-          touched = true;
+      __syncthreads();
+      continue;
+    }
+    // lane l looks at window offset l - 32 (every wave computes the same picture of the window)
+    const int j = lane - kChainLook;
+    int wl = -1;
+    if (j >= jlo && j <= jhi && j != 0) wl = wnear_now;
+    const int fl = tables.b(wl, d).flags;
+    const bool ok = fl != 0 && tables.trained(pa.flags, fl);
+    const unsigned long long valid = __ballot(ok);
+    if (valid == 0ull) continue;
+    const unsigned long long wmask = __ballot(ok && tables.written(fl));
+    const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
+    // A window position belongs to the wave that its place in the token stream selects (so the
+    // same position stays with the same wave while it moves through the windows of consecutive
+    // tokens); a word that stands at several positions of the window belongs, with all of them,
+    // to the wave of its first position, and occurrence number r of it is worked on in round r
+    // (see chain_token_solo).
+    int occ = 0, first = lane;
+    {
+      unsigned long long m = valid;
+      while (m != 0ull) {
+        const int l = __builtin_ctzll(m);
+        m &= m - 1ull;
+        if (l < lane && read_lane(wl, l) == wl) {
+          if (occ == 0) first = l;
+          ++occ;
         }
       }
     }
-    if (touched) {
-      if (tables.written(pa.flags)) atomic_add_col<R>(acol, daa, lane, d);
-      // the adds of this token are performed before the next token's columns are read
+    const bool mine = ok && ((i + first) & (TW - 1)) == wave;
+    const bool repeats = __ballot(ok && occ > 0) != 0ull;
+    float a[R];
+    if (wave == oa) load_col_ordered<R>(a, pa, shadow, 1, chain, lane, d);
+    float daa[R];
+    zero_col<R>(daa);
+    const float ascale = scale_of(wi, vexp, smode);
+
+    int src[CH];
+    int n = 0;
+    float b[CH][R];
+    ColRef rb[CH];
+    auto gather = [&](unsigned long long& mask) {
+      n = 0;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (mask != 0ull) {
+          src[c] = __builtin_ctzll(mask);
+          mask &= mask - 1ull;
+          n = c + 1;
+        } else {
+          src[c] = -1;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (c < n) {
+          rb[c] = tables.b(read_lane(wl, src[c]), d);
+          load_col_ordered<R>(b[c], rb[c], shadow, 0, chain, lane, d);
+        }
+      }
+    };
+    auto update = [&]() {
+      float pre = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (c < n) {
+          const float s = wave_sum(dot_partial<R>(a, b[c]));
+          pre = (lane == c) ? s : pre;
+        }
+      }
+      const float gl = lrate * (1.0f - sat_sigmoid(pre));
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (c < n) {
+          const float g = read_lane(gl, c);
+          const float bs = read_lane(sl, src[c]);
+          axpy<R>(daa, ascale * g, b[c]);
+          if ((wmask >> src[c]) & 1ull) {
+            float db[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) db[r] = (bs * g) * a[r];
+            add_col_ordered<R>(rb[c], shadow, 0, chain, db, lane, d);
+          }
+        }
+      }
+    };
+
+    // the first columns of this wave are requested before the centre's column is handed round
+    unsigned long long mask = __ballot(mine && occ == 0);
+    gather(mask);
+    if (wave == oa) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) s_a[r * kWave + lane] = a[r];
+    }
+    __syncthreads();
+    if (wave != oa) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) a[r] = s_a[r * kWave + lane];
+    }
+    if (n > 0) update();
+    while (mask != 0ull) {
+      gather(mask);
+      update();
+    }
+    for (int round = 1;; ++round) {
+      mask = __ballot(mine && occ == round);
+      if (mask == 0ull) break;
       wait_for_own_writes();
+      while (mask != 0ull) {
+        gather(mask);
+        update();
+      }
+    }
+    // the waves' shares of the centre's delta meet at the centre's owner
+#pragma unroll
+    for (int r = 0; r < R; ++r) s_da[wave][r * kWave + lane] = daa[r];
+    // The next reader of a word that stands at several positions may be another wave (when its
+    // first position leaves the window): this wave's adds have been performed before the team
+    // goes on
+    if (repeats) __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (wave == oa && tables.written(pa.flags)) {
+      zero_col<R>(daa);
+#pragma unroll
+      for (int w = 0; w < TW; ++w) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) daa[r] += s_da[w][r * kWave + lane];
+      }
+      add_col_ordered<R>(pa, shadow, 1, chain, daa, lane, d);
     }
   }
 }
@@ -789,6 +972,18 @@ void set_ordered_workers(int pos, int neg) {
 int ordered_pos_workers() { return g_ordered_pos_workers.load(); }
 int ordered_neg_workers() { return g_ordered_neg_workers.load(); }
 
+// Delta slots of the frequent columns in the ordered kernels: copies x twins.
+static std::atomic<int> g_ordered_copies{2}, g_ordered_twins{2};
+void set_ordered_copies(int copies, int twins) {
+  if (copies < 0 || copies > kGridMaxC || twins < 1 || copies * twins > kShadows) return;
+  g_ordered_copies.store(copies);
+  g_ordered_twins.store(twins);
+}
+void get_ordered_copies(int* copies, int* twins) {
+  *copies = g_ordered_copies.load();
+  *twins = g_ordered_twins.load();
+}
+
 static std::atomic<int> g_hot_update_mode{-1};
 void set_hot_update_mode(int mode) { g_hot_update_mode.store(mode >= 0 && mode <= 2 ? mode : -1); }
 int get_hot_update_mode() { return g_hot_update_mode.load(); }
@@ -815,6 +1010,8 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
     shadow->combine = nwg * waves_per_wg >= kCombineMinWaves ? kHotCombining : kHotExact;
   shadow->combine_a = shadow->combine;
   shadow->ordered = ordered_flag(forced);
+  shadow->grid_c = g_ordered_copies.load();
+  shadow->grid_r = g_ordered_twins.load();
   if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
   if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
@@ -944,19 +1141,19 @@ struct PosChunk {
 };
 
 
-// Workers of the ordered form: as many as keep the missed updates of the most frequent word near
-// what a few dozen CPU threads miss (a lockstep simulation of K workers lands 0.2 %, 0.6 %, 1.4 %,
-// 5 % from the sequential result at K = 16, 32, 128, 256 on a raw Zipf stream), and no fewer
-// than 64 tokens per worker.
-constexpr int kPosChains = 128;
+// Workers of the ordered form, and no fewer than 64 tokens per worker.  What the held-out loss
+// bounds is the tokens that are between their reads and their adds at any time.  Held-out loss of
+// the 10k-vocabulary configuration on a raw stream against the sequential oracle, teams of four
+// waves, 576 negative workers: 96: -0.07 %, 128: -0.06 %, 192: -0.25 %, 256: -0.67 %, 384: -3.1 %;
+// headline shape (8 minibatches, sequential oracle 9.8094): 128: -0.3 %, 192: -0.9 %, 256: -1.7 %.
 constexpr int64_t kMinTokensPerChain = 64;
 
-int64_t ordered_pos_chains(int ncols, int shift) {
+int64_t ordered_pos_chains(int ncols, int shift, int builtin_workers) {
   int64_t chains = ((int64_t)ncols + kMinTokensPerChain - 1) / kMinTokensPerChain;
   // what is bounded is the pairs in flight: a token of a window of half-width 10 has twice the
   // pairs of one of half-width 5, so half the workers
-  int64_t builtin = kPosChains;
-  if (shift > 5) builtin = std::max<int64_t>(32, kPosChains * 6 / (shift + 1));
+  int64_t builtin = builtin_workers;
+  if (shift > 5) builtin = std::max<int64_t>(32, builtin * 6 / (shift + 1));
   const int64_t most = ordered_pos_workers() > 0 ? ordered_pos_workers() : builtin;
   if (chains > most) chains = most;
   const int limit = g_max_workgroups.load();
@@ -964,17 +1161,31 @@ int64_t ordered_pos_chains(int ncols, int shift) {
   return chains < 1 ? 1 : chains;
 }
 
+template <int R, int TW, class Tables>
+static hipError_t launch_pos_chain_tw(hipStream_t stream, int d, int ncols, int64_t chains,
+                                      const int* W, const int* LB, const int* UB,
+                                      const Tables& tables, float lrate, float vexp,
+                                      const Shadow& shadow) {
+  const int64_t per_chain = ((int64_t)ncols + chains - 1) / chains;   // teams beyond: empty range
+  constexpr int CH = TW == 1 ? PosChunk<R>::value : TeamChunk<R>::value;
+  hipLaunchKernelGGL((pos_chain_kernel<R, CH, TW, Tables>), dim3((unsigned)chains),
+                     dim3(kWave * TW), 0, stream, d, ncols, per_chain, W, LB, UB, tables, lrate,
+                     vexp, scale_mode(vexp), shadow);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return launch_grid_fold(stream, tables, shadow, d);
+}
+
 template <int R, class Tables>
 static hipError_t launch_pos_chain(hipStream_t stream, int d, int ncols, int shift, const int* W,
                                    const int* LB, const int* UB, const Tables& tables, float lrate,
                                    float vexp, const Shadow& shadow) {
-  const int64_t chains = ordered_pos_chains(ncols, shift);
-  const int64_t per_chain = ((int64_t)ncols + chains - 1) / chains;   // waves beyond: empty range
-  hipLaunchKernelGGL((pos_chain_kernel<R, PosChunk<R>::value, Tables>),
-                     dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
-                     dim3(kBlock), 0, stream, d, ncols, per_chain, W, LB, UB, tables, lrate, vexp,
-                     scale_mode(vexp), shadow);
-  return hipGetLastError();
+  const int64_t chains = ordered_pos_chains(ncols, shift, kPosTeams);
+  // a window that the 64 lanes of a wave cannot cover is walked by single waves
+  if (shift < kChainLook)
+    return launch_pos_chain_tw<R, kTeamWaves>(stream, d, ncols, chains, W, LB, UB, tables, lrate,
+                                              vexp, shadow);
+  return launch_pos_chain_tw<R, 1>(stream, d, ncols, chains, W, LB, UB, tables, lrate, vexp, shadow);
 }
 
 // Tile size: 16 tokens, or 8 if that is what lets two workgroups share a CU's LDS; if even 8

@@ -365,7 +365,7 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
   err = hipGetLastError();
   if (TRAIN && err == hipSuccess && shadow.ordered != 0)
     err = launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
-                                ordered_neg_chains(kWavesPerBlock), shadow);
+                                ordered_neg_chains(kWavesPerBlock, kNegRowWorkers), shadow);
   return err;
 }
 

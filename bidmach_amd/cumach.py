@@ -75,6 +75,7 @@ SYMBOLS = {
     "w2v_set_ordered_mode": (_I, [_I]),
     "w2v_get_ordered_mode": (_I, []),
     "w2v_set_ordered_workers": (_I, [_I, _I]),
+    "w2v_set_ordered_copies": (_I, [_I, _I]),
     "w2v_set_hot_update_mode": (_I, [_I]),
     "w2v_get_hot_update_mode": (_I, []),
     "w2v_set_rare_update_mode": (_I, [_I]),

@@ -227,6 +227,12 @@ int w2v_get_ordered_mode(void);
  * spreads a launch over; 0 = the library's own numbers (the default).  Fewer workers follow the
  * sequential order more closely and take longer; w2v_set_max_workgroups bounds them as well. */
 int w2v_set_ordered_workers(int pos_workers, int neg_workers);
+/* In the ordered form the columns of the 16 most frequent words are kept, for the length of a
+ * launch, as `copies` x `twins` delta slots next to the (then unchanged) table column: a writer
+ * adds to the `twins` slots of one copy, a reader sums one twin of every copy, so no reader misses
+ * an update and one cache line takes 1/copies of the adds and 1/twins of the reads.  copies <= 8,
+ * copies * twins <= 32; copies = 0: read and update the table columns in place.  Default 4 x 4. */
+int w2v_set_ordered_copies(int copies, int twins);
 
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
  * otherwise serialise the float atomics of the whole device.  No counterpart in the reference.
