@@ -14,7 +14,15 @@ constexpr int kMaxDevices = 64;
 constexpr int kNoIdLimit = 0x7FFFFFFF;
 
 struct ThreadState {
-  hipStream_t stream = nullptr;
+  // The stream the calling thread's launches go to: the caller's (w2v_set_stream), else a stream
+  // of the thread's own per device, created on its first call there.  The reference library is
+  // built with --default-stream per-thread (jni/src/configure:158,196): every JVM thread launches
+  // on a stream of its own that still orders with the legacy default stream, so two learner
+  // threads overlap on the device.  hipStreamCreate's default flags give exactly that kind of
+  // stream (blocking with respect to the null stream, default priority).
+  hipStream_t user = nullptr;
+  bool user_set = false;
+  hipStream_t own[kMaxDevices] = {};
   double* partials[kMaxDevices] = {};
   int64_t capacity[kMaxDevices] = {};
   float* shadow[kMaxDevices] = {};  // two shadow buffers (A then B), zero between calls
@@ -23,6 +31,24 @@ struct ThreadState {
 };
 
 thread_local ThreadState t_state;
+
+// create == false: never creates a stream (for the entry point that may not allocate): the
+// thread's own stream if it exists already, else the legacy default stream.
+hipStream_t launch_stream(bool create = true) {
+  ThreadState& ts = t_state;
+  if (ts.user_set) return ts.user;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (ts.own[dev] == nullptr && create) {
+    hipStream_t s = nullptr;
+    if (hipStreamCreate(&s) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;   // the legacy default stream still works
+    }
+    ts.own[dev] = s;
+  }
+  return ts.own[dev];
+}
 
 std::atomic<double> g_eval_floor{1.0e-40};
 std::atomic<int> g_bf16_hot_words{1024};
@@ -44,7 +70,7 @@ hipError_t side_buffers(int nrows, w2v::HotCols* out) {
   const size_t need = (size_t)2 * w2v::side_columns(n) * w2v::side_stride(nrows);
   if (ts.side16_floats[dev] < need) {
     if (ts.side16[dev] != nullptr) {
-      err = hipStreamSynchronize(ts.stream);
+      err = hipStreamSynchronize(launch_stream());
       if (err != hipSuccess) return err;
       err = hipFree(ts.side16[dev]);
       ts.side16[dev] = nullptr;
@@ -54,8 +80,8 @@ hipError_t side_buffers(int nrows, w2v::HotCols* out) {
     float* p = nullptr;
     err = hipMalloc(reinterpret_cast<void**>(&p), need * sizeof(float));
     if (err != hipSuccess) return err;
-    err = hipMemsetAsync(p, 0, need * sizeof(float), ts.stream);
-    if (err == hipSuccess) err = hipStreamSynchronize(ts.stream);
+    err = hipMemsetAsync(p, 0, need * sizeof(float), launch_stream());
+    if (err == hipSuccess) err = hipStreamSynchronize(launch_stream());
     if (err != hipSuccess) {
       (void)hipFree(p);
       return err;
@@ -77,7 +103,7 @@ hipError_t eval_scratch(int64_t need, double** out) {
   ThreadState& ts = t_state;
   if (ts.capacity[dev] < need) {
     if (ts.partials[dev] != nullptr) {
-      err = hipStreamSynchronize(ts.stream);
+      err = hipStreamSynchronize(launch_stream());
       if (err != hipSuccess) return err;
       err = hipFree(ts.partials[dev]);
       ts.partials[dev] = nullptr;
@@ -113,8 +139,8 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
                          2 * w2v::read_copy_bytes();
     err = hipMalloc(reinterpret_cast<void**>(&p), total);
     if (err != hipSuccess) return err;
-    err = hipMemsetAsync(p, 0, total, ts.stream);
-    if (err == hipSuccess) err = hipStreamSynchronize(ts.stream);  // the stream may change later
+    err = hipMemsetAsync(p, 0, total, launch_stream());
+    if (err == hipSuccess) err = hipStreamSynchronize(launch_stream());  // the stream may change later
     if (err != hipSuccess) {
       (void)hipFree(p);
       return err;
@@ -147,7 +173,7 @@ bool bad_common(int nrows, int ncols) {
 int finish(hipError_t launch_err, bool sync) {
   if (launch_err != hipSuccess) return (int)launch_err;
   if (sync) {
-    hipError_t err = hipStreamSynchronize(t_state.stream);
+    hipError_t err = hipStreamSynchronize(launch_stream());
     if (err != hipSuccess) return (int)err;
     return (int)hipGetLastError();
   }
@@ -162,7 +188,7 @@ int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp,
+  return finish(w2v::launch_pos(launch_stream(), nrows, ncols, shift, W, LB, UB, A, B, lrate, vexp,
                                 shadow),
                 sync);
 }
@@ -176,7 +202,7 @@ int neg_impl(int nrows, int ncols, int idlimit, int nwa, int nwb, int* WA, int* 
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_neg(t_state.stream, nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B,
+  return finish(w2v::launch_neg(launch_stream(), nrows, ncols, idlimit, nwa, nwb, WA, WB, A, B,
                                 lrate, vexp, shadow),
                 sync);
 }
@@ -189,7 +215,7 @@ int eval_pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, floa
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_eval_pos(t_state.stream, nrows, ncols, W, LB, UB, A, B,
+  return finish(w2v::launch_eval_pos(launch_stream(), nrows, ncols, W, LB, UB, A, B,
                                      g_eval_floor.load(), partials, r32, r64),
                 sync);
 }
@@ -203,7 +229,7 @@ int eval_neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, floa
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+  return finish(w2v::launch_eval_neg(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, A, B,
                                      g_eval_floor.load(), partials, r32, r64),
                 sync);
 }
@@ -246,7 +272,7 @@ int pos_slice_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, fl
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_slice_pos(t_state.stream, nrows, ncols, shift, W, LB, UB, m, lrate,
+  return finish(w2v::launch_slice_pos(launch_stream(), nrows, ncols, shift, W, LB, UB, m, lrate,
                                       vexp, shadow),
                 true);
 }
@@ -263,7 +289,7 @@ int neg_slice_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, flo
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_slice_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, m, lrate,
+  return finish(w2v::launch_slice_neg(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, m, lrate,
                                       vexp, shadow),
                 true);
 }
@@ -280,7 +306,7 @@ int eval_pos_slice_impl(int nrows, int ncols, int* W, int* LB, int* UB, float** 
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::slice_eval_partials_needed(), &partials);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_slice_eval_pos(t_state.stream, nrows, ncols, W, LB, UB, m,
+  return finish(w2v::launch_slice_eval_pos(launch_stream(), nrows, ncols, W, LB, UB, m,
                                            g_eval_floor.load(), partials, nullptr, Retval),
                 true);
 }
@@ -297,7 +323,7 @@ int eval_neg_slice_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::slice_eval_partials_needed(), &partials);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_slice_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, m,
+  return finish(w2v::launch_slice_eval_neg(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, m,
                                            g_eval_floor.load(), partials, nullptr, Retval),
                 true);
 }
@@ -413,11 +439,16 @@ int word2vecEvalNegNoAlloc(int nrows, int ncols, int nwa, int nwb, int* WA, int*
   hipError_t err = static_scratch(&partials);
   if (err != hipSuccess) return (int)err;
   // every workgroup overwrites its own partial sum and the fold reads only those: nothing in
-  // the array has to start at zero
-  return finish(w2v::launch_eval_neg(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
-                                     g_eval_floor.load(), partials, Retval, nullptr,
-                                     kStaticPartials),
-                true);
+  // the array has to start at zero.  The stream is the caller's, or the thread's own if an
+  // earlier call created it, else the legacy default stream: none is created here.
+  hipStream_t stream = launch_stream(false);
+  hipError_t lerr = w2v::launch_eval_neg(stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+                                         g_eval_floor.load(), partials, Retval, nullptr,
+                                         kStaticPartials);
+  if (lerr != hipSuccess) return (int)lerr;
+  lerr = hipStreamSynchronize(stream);
+  if (lerr != hipSuccess) return (int)lerr;
+  return (int)hipGetLastError();
 }
 
 int w2v_no_alloc_max_groups(void) { return kNoAllocMaxGroups; }
@@ -468,7 +499,7 @@ static int pos_bf16_impl(int nrows, int ncols, int shift, int* W, int* LB, int* 
   w2v::Shadow shadow{};   // for its hot-word counters: the launch may run in its ordered form
   err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_pos_bf16(t_state.stream, nrows, ncols, shift, W, LB, UB, A, B, lrate,
+  return finish(w2v::launch_pos_bf16(launch_stream(), nrows, ncols, shift, W, LB, UB, A, B, lrate,
                                      vexp, seed, hot, shadow),
                 sync);
 }
@@ -497,7 +528,7 @@ static int neg_bf16_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* W
   w2v::Shadow shadow{};
   err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
-  return finish(w2v::launch_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
+  return finish(w2v::launch_neg_bf16(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, A, B, lrate,
                                      vexp, seed, hot, shadow),
                 sync);
 }
@@ -519,7 +550,7 @@ int word2vecEvalPosBf16(int nrows, int ncols, int shift, int* W, int* LB, int* U
   if (bad_common(nrows, ncols) || !Retval) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_eval_pos_bf16(t_state.stream, nrows, ncols, W, LB, UB, A, B,
+  return finish(w2v::launch_eval_pos_bf16(launch_stream(), nrows, ncols, W, LB, UB, A, B,
                                           g_eval_floor.load(), Retval),
                 true);
 }
@@ -530,7 +561,7 @@ int word2vecEvalNegBf16(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_eval_neg_bf16(t_state.stream, nrows, ncols, nwa, nwb, WA, WB, A, B,
+  return finish(w2v::launch_eval_neg_bf16(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, A, B,
                                           g_eval_floor.load(), Retval),
                 true);
 }
@@ -545,32 +576,46 @@ int w2v_get_bf16_hot_words(void) { return g_bf16_hot_words.load(); }
 int w2v_f32_to_bf16(size_t n, const float* src, unsigned short* dst) {
   if (n == 0) return 0;
   if (!src || !dst) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_f32_to_bf16(t_state.stream, n, src, dst), true);
+  return finish(w2v::launch_f32_to_bf16(launch_stream(), n, src, dst), true);
 }
 
 int w2v_bf16_to_f32(size_t n, const unsigned short* src, float* dst) {
   if (n == 0) return 0;
   if (!src || !dst) return (int)hipErrorInvalidValue;
-  return finish(w2v::launch_bf16_to_f32(t_state.stream, n, src, dst), true);
+  return finish(w2v::launch_bf16_to_f32(launch_stream(), n, src, dst), true);
 }
 
 void w2v_set_eval_floor(double floor_value) { g_eval_floor.store(floor_value); }
 double w2v_get_eval_floor(void) { return g_eval_floor.load(); }
 
 int w2v_set_stream(void* stream) {
-  t_state.stream = reinterpret_cast<hipStream_t>(stream);
+  t_state.user = reinterpret_cast<hipStream_t>(stream);
+  t_state.user_set = true;
   return 0;
 }
-void* w2v_get_stream(void) { return reinterpret_cast<void*>(t_state.stream); }
-int w2v_synchronize(void) { return (int)hipStreamSynchronize(t_state.stream); }
+int w2v_reset_stream(void) {
+  t_state.user = nullptr;
+  t_state.user_set = false;
+  return 0;
+}
+void* w2v_get_stream(void) { return reinterpret_cast<void*>(launch_stream()); }
+int w2v_synchronize(void) { return (int)hipStreamSynchronize(launch_stream()); }
 
 int w2v_release_thread(void) {
   ThreadState& ts = t_state;
   bool held = false;
   for (int dev = 0; dev < kMaxDevices; ++dev)
-    held = held || ts.partials[dev] || ts.shadow[dev] || ts.side16[dev];
+    held = held || ts.partials[dev] || ts.shadow[dev] || ts.side16[dev] || ts.own[dev];
   if (!held) return 0;
-  hipError_t first = hipStreamSynchronize(ts.stream);   // nothing may still be using the scratch
+  hipError_t first = hipStreamSynchronize(launch_stream(false));   // nothing may still be using the scratch
+  for (int dev = 0; dev < kMaxDevices; ++dev) {
+    if (ts.own[dev] != nullptr) {
+      hipError_t err = hipStreamSynchronize(ts.own[dev]);
+      if (err == hipSuccess) err = hipStreamDestroy(ts.own[dev]);
+      if (first == hipSuccess) first = err;
+      ts.own[dev] = nullptr;
+    }
+  }
   auto release = [&first](auto*& p) {
     if (p != nullptr) {
       const hipError_t err = hipFree(p);
@@ -633,19 +678,19 @@ int w2v_malloc(void** dev_ptr, size_t bytes) {
 }
 int w2v_free(void* dev_ptr) { return (int)hipFree(dev_ptr); }
 int w2v_memcpy_h2d(void* dev_dst, const void* host_src, size_t bytes) {
-  hipError_t err = hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, t_state.stream);
+  hipError_t err = hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, launch_stream());
   if (err != hipSuccess) return (int)err;
-  return (int)hipStreamSynchronize(t_state.stream);
+  return (int)hipStreamSynchronize(launch_stream());
 }
 int w2v_memcpy_d2h(void* host_dst, const void* dev_src, size_t bytes) {
-  hipError_t err = hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, t_state.stream);
+  hipError_t err = hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, launch_stream());
   if (err != hipSuccess) return (int)err;
-  return (int)hipStreamSynchronize(t_state.stream);
+  return (int)hipStreamSynchronize(launch_stream());
 }
 int w2v_memset(void* dev_ptr, int value, size_t bytes) {
-  hipError_t err = hipMemsetAsync(dev_ptr, value, bytes, t_state.stream);
+  hipError_t err = hipMemsetAsync(dev_ptr, value, bytes, launch_stream());
   if (err != hipSuccess) return (int)err;
-  return (int)hipStreamSynchronize(t_state.stream);
+  return (int)hipStreamSynchronize(launch_stream());
 }
 
 int w2v_timer_create(void** timer) {
@@ -676,11 +721,11 @@ int w2v_timer_destroy(void* timer) {
 }
 int w2v_timer_start(void* timer) {
   if (!timer) return (int)hipErrorInvalidValue;
-  return (int)hipEventRecord(static_cast<Timer*>(timer)->start, t_state.stream);
+  return (int)hipEventRecord(static_cast<Timer*>(timer)->start, launch_stream());
 }
 int w2v_timer_stop(void* timer) {
   if (!timer) return (int)hipErrorInvalidValue;
-  return (int)hipEventRecord(static_cast<Timer*>(timer)->stop, t_state.stream);
+  return (int)hipEventRecord(static_cast<Timer*>(timer)->stop, launch_stream());
 }
 int w2v_timer_elapsed_ms(void* timer, float* ms) {
   if (!timer || !ms) return (int)hipErrorInvalidValue;

@@ -223,9 +223,11 @@ struct Shadow {
   float* b;         // same for table B
   unsigned* count;  // [2][kShadows][kHotWords][kCounterStride] write counters (B then A); they
                     // only ever count up, so they need no clearing between calls
-  // Counted on the device before the launch, kHotCountSlots partial counts each: how many of the
-  // hot_total word ids read from table B are below kHotWords, how many are 0, and the same two
-  // for the hot_total_a ids read from table A (0: table A follows table B).  hot_total == 0: not
+  // Counted on the device before the launch (count_heavy_kernel), kHotCountSlots partial counts
+  // each: how many of the hot_total word ids read from table B belong to the kHotWords most
+  // frequent words of the launch, how many to the most frequent one, and the same two for the
+  // hot_total_a ids read from table A (0: table A follows table B).  The counts are of
+  // occurrences, so they do not depend on how the vocabulary is numbered.  hot_total == 0: not
   // counted, the modes below stand.
   int* hot_seen;
   long long hot_total;
@@ -281,10 +283,10 @@ __device__ __forceinline__ long long sum_hot_counts(const int* part) {
   return __builtin_amdgcn_readfirstlane(t);
 }
 
-// Whether `total` word ids with `low` of them below kHotWords and `zero` of them equal to 0 are
-// worth shadow copies: the 16 lowest ids are a sixteenth of all, or id 0 alone is a 48th (its
-// atomics retire one after the other, and at 5 ids per group a 48th of them already lasts about
-// half as long as the whole pass).
+// Whether `total` word ids, `low` of them occurrences of the kHotWords most frequent words and
+// `zero` of them of the most frequent one, are full of frequent words: the 16 most frequent are a
+// sixteenth of all, or the most frequent alone is a 48th (its atomics retire one after the other,
+// and at 5 ids per group a 48th of them already lasts about half as long as the whole pass).
 __device__ __forceinline__ bool ids_are_hot(long long low, long long zero, long long total) {
   return low * kHotShareDen >= total || zero * kHotZeroShareDen >= total;
 }
@@ -316,11 +318,15 @@ __device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow
          resolved.combine_a == kHotOff;
 }
 
-// Waits until this wave's outstanding memory operations, its float atomics and exchanges among
-// them, have been performed.  The ordered kernels call it between a worker's writes and the reads
-// that must see them.  All their writes are device-scope atomics, performed at the memory side, so
-// there is nothing in a cache to write back: the fence is of workgroup scope, which is the wait
-// alone (an agent-scope release adds a write-back of the XCD's L2, 6 ms per 1M-token pass).
+// Keeps the compiler from moving a worker's later reads above its earlier adds.  It is NOT a
+// wait: a workgroup-scope release fence emits no s_waitcnt on this target.  What the ordered
+// kernels rely on is that requests of one wave to one address are performed in the order they
+// were issued (a device-scope load that follows a device-scope atomic add of the same wave to the
+// same address returns the sum), which the one-worker sequential-equivalence tests pin; a real
+// wait for the adds' acknowledgements is __builtin_amdgcn_s_waitcnt(0), which the team kernel uses
+// where the next reader of a column may be another wave.  (An agent-scope release fence adds a
+// write-back of the XCD's L2, 6 ms per 1M-token pass, for nothing: every write of these kernels
+// is a device-scope atomic, performed at the memory side.)
 __device__ __forceinline__ void wait_for_own_writes() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
 }

@@ -4,7 +4,8 @@
 //
 // Semantics are those of BIDMach_CPUMACH.c:186-264: every dot of a group uses the A columns as
 // they were when the group started (A is written after the group's last dot, :248-254) and a B
-// column as it was when its own row started.  Walking the B columns in tiles and re-reading A for
+// column as it was when its own tile of rows started (read with device-scope loads, so that a
+// word of an earlier tile is seen as that tile's adds left it).  Walking the B columns in tiles and re-reading A for
 // every tile would break the first rule (a later tile would see the deltas of the earlier ones,
 // an error of the order of the squared step, which is not small for the large steps that
 // vexp > 0 gives rare words).  So the group's A columns are staged once, in LDS, next to an fp32
@@ -35,14 +36,33 @@ __device__ __forceinline__ void load_col_any(float (&x)[R], const float* col, in
   }
 }
 
+// The same with device-scope loads, for the B columns: a B word that occurs in two tiles of one
+// group (or in two groups of this workgroup) was updated with a device-scope add, which a plain
+// load could still answer from this CU's L1 with the value from before.
+template <int R>
+__device__ __forceinline__ void load_col_any_fresh(float (&x)[R], const float* col, int lane,
+                                                   int d) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int e = r * kWave + lane;
+    x[r] = e < d ? __hip_atomic_load(col + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+  }
+}
+
 // R here is an upper bound of ceil(d / 64): rounds beyond d hold zeros and are never stored.
 template <int R, int MAXB, typename Tables>
 __global__ void __launch_bounds__(kWave)
-neg_wide_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_wg,
-                const int* __restrict__ WA, const int* __restrict__ WB, Tables tables, float lrate,
+neg_wide_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_wg_all,
+                int64_t per_wg_ordered, const int* __restrict__ WA, const int* __restrict__ WB,
+                Tables tables, float lrate,
                 float vexp, int smode, Shadow shadow_arg) {
-  // a launch full of frequent words is done by neg_rows_kernel (launch_is_ordered, w2v_device.h)
-  if (shadow_arg.ordered != 0 && launch_is_ordered(shadow_arg, resolve_hot_mode(shadow_arg))) return;
+  // a launch full of frequent words is done by neg_rows_kernel (launch_is_ordered, w2v_device.h),
+  // or, where that has no instance for the shape, by this kernel on a few workgroups
+  int64_t per_wg = per_wg_all;
+  if (shadow_arg.ordered != 0 && launch_is_ordered(shadow_arg, resolve_hot_mode(shadow_arg))) {
+    if (per_wg_ordered == 0) return;
+    per_wg = per_wg_ordered;
+  }
   extern __shared__ float lds[];
   constexpr int RS = R * kWave;
   float* const a_old = lds;                          // [nwa][RS]
@@ -98,7 +118,7 @@ neg_wide_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_w
           fb[k] = read_lane(pbl.flags, kb + k);
           if (fb[k] != 0) {
             bcol[k] = tables.b(read_lane(wbl, kb + k), d).col;
-            load_col_any<R>(b[k], bcol[k], lane, d);
+            load_col_any_fresh<R>(b[k], bcol[k], lane, d);
           }
         }
         zero_col<R>(dbb[k]);
@@ -153,6 +173,9 @@ neg_wide_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_w
 }
 
 constexpr int64_t kWideMinGroupsPerWg = 64;
+// workgroups (of one wave) that run an ordered launch whose shape the row-by-row kernel has no
+// instance for: the group-at-a-time order needs 32 or fewer workers for 1 % of held-out loss
+constexpr int64_t kWideOrderedWorkers = 32;
 
 template <int R, typename Tables>
 hipError_t launch_wide_r(hipStream_t stream, int d, int ngroups, int idlimit, int nwa, int nwb,
@@ -181,11 +204,17 @@ hipError_t launch_wide_r(hipStream_t stream, int d, int ngroups, int idlimit, in
     err = prepare_hot_mode(stream, WB, (int64_t)ngroups * nwb, WA, (int64_t)ngroups * nwa, nullptr,
                            nullptr, d, nwg, 1, &shadow);
   if (err != hipSuccess) return err;
-  if (!neg_rows_available(d, nwa)) shadow.ordered = 0;
+  const bool rows = shadow.ordered != 0 && neg_rows_available(d, nwa);
+  int64_t per_wg_ordered = 0;
+  if (shadow.ordered != 0 && !rows) {
+    const int64_t wgs = nwg < kWideOrderedWorkers ? nwg : kWideOrderedWorkers;
+    per_wg_ordered = ((int64_t)ngroups + wgs - 1) / wgs;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kWave), lds, stream, d, ngroups, idlimit,
-                     nwa, nwb, per_wg, WA, WB, tables, lrate, vexp, scale_mode(vexp), shadow);
+                     nwa, nwb, per_wg, per_wg_ordered, WA, WB, tables, lrate, vexp,
+                     scale_mode(vexp), shadow);
   err = hipGetLastError();
-  if (err != hipSuccess || shadow.ordered == 0) return err;
+  if (err != hipSuccess || !rows) return err;
   if constexpr (Tables::kSliced)
     return launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, tables.m, lrate, vexp,
                                  ordered_neg_chains(kWavesPerBlock, kNegRowWorkers), shadow);

@@ -826,22 +826,102 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
   }
 }
 
-// Counts the word ids below kHotWords, and those equal to 0, among `ids` and among `ids2`: block b
-// leaves its four shares in out[k * kHotCountSlots + b] (kHotCountSlots blocks, every slot is
-// written on every launch, so nothing needs clearing and no atomics queue up).  It also leaves, in mask[b] and mask[kHotCountSlots + b], bit masks of the hot
-// ids it saw in `ids` (the words read from table B) and in `ids2` (those read from table A; null:
-// the same as `ids`); there a word counts under the index of its shadow copies (ColRef::hot), which
-// for a sliced model is its packed column and not its id.
+// How full of frequent words a launch is, whatever the numbering of the vocabulary: a sample of
+// at most kHeavySamples ids of `ids` (the words read from table B) is counted into a hashed
+// histogram in LDS, and the sum of its kHeavyTop largest bins and its largest bin, scaled up to
+// the n ids of the launch, are left where the update kernels look for "the ids among the 16 most
+// frequent words" and "the most frequent word" (Shadow::hot_seen: four arrays of kHotCountSlots
+// partial counts; the values go to slot 0, the other slots are zeroed); the same for `ids2` (the
+// words read from table A; null: not counted).  Two frequent words that share a bin only make the
+// largest bin larger, and the words that are not frequent add about four ids to every bin, 0.4 %
+// of the sample over the kHeavyTop bins: both err towards "frequent".  One workgroup.
+constexpr int kHeavyThreads = 1024;
+constexpr int kHeavySamples = 16384;
+constexpr int kHeavyBins = 4096;
+constexpr int kHeavyTop = kHotWords;
+__global__ void __launch_bounds__(kHeavyThreads)
+count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
+                   int* __restrict__ out) {
+  __shared__ int s_bins[kHeavyBins];
+  __shared__ int s_val[kHeavyThreads / kWave], s_idx[kHeavyThreads / kWave];
+  __shared__ int s_pick;
+  const int tid = threadIdx.x;
+  for (int which = 0; which < 2; ++which) {
+    const int* const p = which ? ids2 : ids;
+    const int64_t len = which ? n2 : n;
+    long long top_sum = 0, top_one = 0;
+    if (p != nullptr && len > 0) {
+      for (int k = tid; k < kHeavyBins; k += kHeavyThreads) s_bins[k] = 0;
+      __syncthreads();
+      const int64_t stride = (len + kHeavySamples - 1) / kHeavySamples;
+      const int64_t nsamp = (len + stride - 1) / stride;
+      for (int64_t k = tid; k < nsamp; k += kHeavyThreads) {
+        const int w = p[k * stride];
+        if (w >= 0) atomicAdd(&s_bins[((unsigned)w * 2654435761u) >> 20], 1);
+      }
+      __syncthreads();
+      for (int round = 0; round < kHeavyTop; ++round) {
+        int best = -1, at = 0;
+        for (int k = tid; k < kHeavyBins; k += kHeavyThreads) {
+          const int v = s_bins[k];
+          if (v > best) {
+            best = v;
+            at = k;
+          }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+          const int ov = __shfl_xor(best, m, kWave), oi = __shfl_xor(at, m, kWave);
+          if (ov > best || (ov == best && oi < at)) {
+            best = ov;
+            at = oi;
+          }
+        }
+        if ((tid & 63) == 0) {
+          s_val[tid >> 6] = best;
+          s_idx[tid >> 6] = at;
+        }
+        __syncthreads();
+        if (tid == 0) {
+          int bv = -1, bi = 0;
+          for (int k = 0; k < kHeavyThreads / kWave; ++k) {
+            if (s_val[k] > bv) {
+              bv = s_val[k];
+              bi = s_idx[k];
+            }
+          }
+          s_pick = bv;
+          s_bins[bi] = 0;
+        }
+        __syncthreads();
+        top_sum += s_pick;
+        if (round == 0) top_one = s_pick;
+      }
+      // sampled counts scaled up to the whole array (dropped words, id < 0, stay in the total)
+      top_sum = top_sum * len / nsamp;
+      top_one = top_one * len / nsamp;
+    }
+    for (int k = tid; k < kHotCountSlots; k += kHeavyThreads) {
+      out[(2 * which) * kHotCountSlots + k] = k == 0 ? (int)min(top_sum, (long long)0x7fffffff) : 0;
+      out[(2 * which + 1) * kHotCountSlots + k] = k == 0 ? (int)min(top_one, (long long)0x7fffffff) : 0;
+    }
+    __syncthreads();
+  }
+}
+
+// Leaves, in mask[b] and mask[kHotCountSlots + b] (kHotCountSlots blocks), bit masks of the ids
+// below kHotWords that block b saw in `ids` (the words read from table B) and in `ids2` (those
+// read from table A; null: the same as `ids`): the columns that may have shadow copies, read
+// copies or delta slots in this launch.  There a word counts under the index of its shadow
+// copies (ColRef::hot), which for a sliced model is its packed column and not its id.  Every slot
+// is written on every launch, so nothing needs clearing.
 template <class Tables>
 __global__ void __launch_bounds__(kBlock)
 count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
-                 Tables tables, int* __restrict__ out, int* __restrict__ mask) {
-  __shared__ int s_part[4][kWavesPerBlock], s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
-  int local = 0, zero = 0, local2 = 0, zero2 = 0, seen = 0, seen2 = 0;
-  // low 16 bits: 1 for an id below kHotWords; high 16 bits: 1 for id 0 (a thread sees far fewer
-  // than 65536 ids)
-  auto hot = [](int w) { return ((w >= 0 && w < kHotWords) ? 1 : 0) + (w == 0 ? 0x10000 : 0); };
-  auto scan = [&](const int* p, int64_t len, int& count, int& bits, bool of_a) {
+                 Tables tables, int* __restrict__ mask) {
+  __shared__ int s_mask[kWavesPerBlock], s_mask2[kWavesPerBlock];
+  int seen = 0, seen2 = 0;
+  auto scan = [&](const int* p, int64_t len, int& bits, bool of_a) {
     auto bit = [&](int w) {
       if (Tables::kSliced) {
         const int h = w >= 0 ? (of_a ? tables.a(w, 0).hot : tables.b(w, 0).hot) : -1;
@@ -856,50 +936,29 @@ count_hot_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__
       for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < len4;
            i += (int64_t)gridDim.x * kBlock) {
         const int4 v = p4[i];
-        count += hot(v.x) + hot(v.y) + hot(v.z) + hot(v.w);
         bits |= bit(v.x) | bit(v.y) | bit(v.z) | bit(v.w);
       }
     }
     for (int64_t i = (aligned ? len4 * 4 : 0) + (int64_t)blockIdx.x * kBlock + threadIdx.x;
-         i < len; i += (int64_t)gridDim.x * kBlock) {
-      count += hot(p[i]);
+         i < len; i += (int64_t)gridDim.x * kBlock)
       bits |= bit(p[i]);
-    }
   };
-  scan(ids, n, local, seen, false);
+  scan(ids, n, seen, false);
   if (ids2 != nullptr || Tables::kSliced) {
-    scan(ids2 != nullptr ? ids2 : ids, ids2 != nullptr ? n2 : n, local2, seen2, true);
+    scan(ids2 != nullptr ? ids2 : ids, ids2 != nullptr ? n2 : n, seen2, true);
   } else {
     seen2 = seen;
   }
-  zero = local >> 16;
-  local &= 0xffff;
-  zero2 = local2 >> 16;
-  local2 &= 0xffff;
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) {
-    local += __shfl_xor(local, m, kWave);
-    zero += __shfl_xor(zero, m, kWave);
-    local2 += __shfl_xor(local2, m, kWave);
-    zero2 += __shfl_xor(zero2, m, kWave);
     seen |= __shfl_xor(seen, m, kWave);
     seen2 |= __shfl_xor(seen2, m, kWave);
   }
   if ((threadIdx.x & 63) == 0) {
-    s_part[0][threadIdx.x >> 6] = local;
-    s_part[1][threadIdx.x >> 6] = zero;
-    s_part[2][threadIdx.x >> 6] = local2;
-    s_part[3][threadIdx.x >> 6] = zero2;
     s_mask[threadIdx.x >> 6] = seen;
     s_mask2[threadIdx.x >> 6] = seen2;
   }
   __syncthreads();
-  if (threadIdx.x < 4) {
-    int total = 0;
-#pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[threadIdx.x][w];
-    out[threadIdx.x * kHotCountSlots + blockIdx.x] = total;
-  }
   if (threadIdx.x == 0) {
     int m1 = 0, m2 = 0;
 #pragma unroll
@@ -1018,7 +1077,9 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   // read the count from memory, the host does not wait for it).  The same pass notes which hot
   // ids occur at all, for the read copies.
   hipLaunchKernelGGL(count_hot_kernel<Tables>, dim3(kHotCountSlots), dim3(kBlock), 0, stream, ids,
-                     n, ids2, n2, tables, shadow->hot_seen, shadow->hot_mask);
+                     n, ids2, n2, tables, shadow->hot_mask);
+  hipLaunchKernelGGL(count_heavy_kernel, dim3(1), dim3(kHeavyThreads), 0, stream, ids, n, ids2, n2,
+                     shadow->hot_seen);
   if (!forced) {
     shadow->hot_total = n;
     shadow->hot_total_a = ids2 != nullptr ? n2 : 0;

@@ -137,13 +137,17 @@ slice_pos_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__
 
 template <int R, int MAXB, int CHA, bool TRAIN>
 __global__ void __launch_bounds__(kBlock, 3)
-slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg,
-                 const int* __restrict__ WA, const int* __restrict__ WB, SlicedTables tables,
+slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg_all,
+                 int64_t units_per_wg_ordered, const int* __restrict__ WA, const int* __restrict__ WB, SlicedTables tables,
                  float lrate, float vexp, int smode, double floorv, double* __restrict__ partials,
                  Shadow shadow_arg) {
   static_assert(MAXB * CHA <= kWave, "one lane per pre-activation of a chunk");
   const Shadow shadow = TRAIN ? resolve_hot_mode(shadow_arg) : shadow_arg;
-  if (TRAIN && launch_is_ordered(shadow_arg, shadow)) return;   // neg_rows_kernel does this launch
+  int64_t units_per_wg = units_per_wg_all;
+  if (TRAIN && launch_is_ordered(shadow_arg, shadow)) {
+    if (units_per_wg_ordered == 0) return;    // neg_rows_kernel does this launch
+    units_per_wg = units_per_wg_ordered;      // no ordered instance for this shape: few workers
+  }
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = blockIdx.x;
@@ -355,15 +359,21 @@ static hipError_t launch_slice_neg_rb(hipStream_t stream, int d, int ngroups, in
     err = prepare_rare_words(stream, WA, (int64_t)ngroups * nwa, WB, (int64_t)ngroups * nwb,
                              0x7fffffff, ngroups, nwg * kWavesPerBlock, &shadow);
     if (err != hipSuccess) return err;
-    // ordered launches go to the row-by-row kernel where it has an instance for the shape
-    if (!neg_rows_available(d, nwa)) shadow.ordered = 0;
+  }
+  // ordered launches go to the row-by-row kernel where it has an instance for the shape, else
+  // this kernel runs them on a few workgroups (8 x 4 waves, as the single-table operator does)
+  const bool rows = TRAIN && shadow.ordered != 0 && neg_rows_available(d, nwa);
+  int64_t per_wg_ordered = 0;
+  if (TRAIN && shadow.ordered != 0 && !rows) {
+    const int64_t wgs = nwg < 8 ? nwg : 8;
+    per_wg_ordered = ((int64_t)ngroups + wgs - 1) / wgs;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBlock), 0, stream, d, ngroups, nwa, nwb,
-                     per_wg, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp), floorv, partials,
-                     shadow);
+                     per_wg, per_wg_ordered, WA, WB, SlicedTables{m}, lrate, vexp, scale_mode(vexp),
+                     floorv, partials, shadow);
   *nparts = nwg;
   err = hipGetLastError();
-  if (TRAIN && err == hipSuccess && shadow.ordered != 0)
+  if (err == hipSuccess && rows)
     err = launch_slice_neg_rows(stream, d, ngroups, nwa, nwb, WA, WB, m, lrate, vexp,
                                 ordered_neg_chains(kWavesPerBlock, kNegRowWorkers), shadow);
   return err;

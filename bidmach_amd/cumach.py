@@ -67,6 +67,7 @@ SYMBOLS = {
     "w2v_set_eval_floor": (None, [_D]),
     "w2v_get_eval_floor": (_D, []),
     "w2v_set_stream": (_I, [_P]),
+    "w2v_reset_stream": (_I, []),
     "w2v_get_stream": (_P, []),
     "w2v_synchronize": (_I, []),
     "w2v_release_thread": (_I, []),

@@ -17,7 +17,10 @@
  *
  * Threading (reference: MatKernel.hpp:2 and the per-thread default stream of its build): the
  * four reference calls block until the work is done.  Each host thread has its own launch stream
- * (the null stream until w2v_set_stream is called) and its own Eval scratch buffer.
+ * (one the library creates on the thread's first call on a device, ordered with the legacy
+ * default stream as the reference's per-thread default streams are, jni/src/configure:158,196;
+ * w2v_set_stream replaces it) and its own Eval scratch buffer, so calls from two threads overlap
+ * on the device.
  */
 #ifndef BIDMACH_W2V_H_
 #define BIDMACH_W2V_H_
@@ -105,12 +108,15 @@ int word2vecEvalPosF64(int nrows, int ncols, int shift, int *W, int *LB, int *UB
 int word2vecEvalNegF64(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A,
                        float *B, double *Retval);
 
-/* word2vecEvalNeg for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
- * Same arguments and the same result as word2vecEvalNeg (added into the device float Retval[0];
- * blocking), but the per-workgroup partial sums go to a 64 KB array that is part of the library's
- * device code instead of a buffer taken from hipMalloc on a thread's first call, and the call
- * makes no hipMalloc, hipFree or other allocating call.  At most w2v_no_alloc_max_groups()
+/* word2vecEvalNeg for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc, hosts that score between the captures of a HIP graph).  It has no
+ * counterpart in the reference.  Same arguments and the same result as word2vecEvalNeg (added
+ * into the device float Retval[0]).  Like it, the call blocks until the sum is there (it ends in
+ * a stream synchronisation), so it cannot itself be recorded into a graph.  The per-workgroup
+ * partial sums go to a 64 KB array that is part of the library's device code instead of a buffer
+ * taken from hipMalloc on a thread's first call, and the call makes no hipMalloc, hipFree or
+ * other allocating call; it creates no stream either (it launches on the caller's stream, on the
+ * thread's own if an earlier call made one, else on the legacy default stream).  At most w2v_no_alloc_max_groups()
  * (16,777,216) groups per call; more is rejected with hipErrorInvalidValue.  Every call on a GPU
  * uses that GPU's one array: calls that overlap in time on one GPU (from several threads or
  * streams) race and return wrong sums; one after the other they are independent (nothing in the
@@ -183,15 +189,18 @@ int w2v_bf16_to_f32(size_t n, const unsigned short *src, float *dst);
 void w2v_set_eval_floor(double floor_value);
 double w2v_get_eval_floor(void);
 
-/* Launch stream of the calling thread (a hipStream_t passed as void*; NULL = the null stream). */
+/* Launch stream of the calling thread.  w2v_set_stream: a hipStream_t passed as void* (NULL = the
+ * legacy default stream); w2v_reset_stream: back to the thread's own stream; w2v_get_stream: the
+ * stream the next call will launch on (creates the thread's own stream if there is none yet). */
 int w2v_set_stream(void *stream);
+int w2v_reset_stream(void);
 void *w2v_get_stream(void);
 int w2v_synchronize(void);
 
 /* Frees the device scratch memory the calling thread holds (per device: the forward sums'
  * partial buffer, the shadow and occurrence-count buffers of the update operators, the fp32 side
- * buffers of the bfloat16 operators; allocated on the thread's first calls) after waiting for the
- * thread's launch stream.  The next call allocates it again.  Call it before a worker thread that
+ * buffers of the bfloat16 operators; allocated on the thread's first calls) and destroys the
+ * thread's own launch streams, after waiting for them.  The next call allocates it again.  Call it before a worker thread that
  * used the library ends (a JVM thread pool, say): thread-local scratch is not freed by thread
  * exit.  No counterpart in the reference, whose launchers keep no state. */
 int w2v_release_thread(void);
@@ -216,10 +225,11 @@ int w2v_get_max_workgroups(void);
  * a few hundred wavefronts each walk a contiguous range of tokens / groups in the reference's
  * order, with every column read afresh and every B delta added before the next read.
  *  -1  (default) decided per launch on the device, by the same count that decides about shadow
- *      copies below: ordered if at least 1/16 of the word ids of the launch are among the 16
- *      lowest, or at least 1/48 are id 0; launches without frequent words (after the reference
- *      caller's subsampling, Word2Vec.scala:221-225) keep the throughput kernels.  A forced
- *      w2v_set_hot_update_mode also keeps them.
+ *      copies below: ordered if at least 1/16 of the word ids of the launch are occurrences of
+ *      its 16 most frequent words, or at least 1/48 of its most frequent word (counted on a
+ *      sample of the launch's ids, whatever the numbering of the vocabulary); launches without
+ *      frequent words (after the reference caller's subsampling, Word2Vec.scala:221-225) keep
+ *      the throughput kernels.  A forced w2v_set_hot_update_mode also keeps them.
  *   0  never;  1  always. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
@@ -231,7 +241,8 @@ int w2v_set_ordered_workers(int pos_workers, int neg_workers);
  * launch, as `copies` x `twins` delta slots next to the (then unchanged) table column: a writer
  * adds to the `twins` slots of one copy, a reader sums one twin of every copy, so no reader misses
  * an update and one cache line takes 1/copies of the adds and 1/twins of the reads.  copies <= 8,
- * copies * twins <= 32; copies = 0: read and update the table columns in place.  Default 4 x 4. */
+ * copies * twins <= 32; copies = 0: read and update the table columns in place.  Default 2 x 2.
+ * The 16 columns are those of ids 0..15: the slots pay when ids are frequency ranks. */
 int w2v_set_ordered_copies(int copies, int twins);
 
 /* How the update operators treat the few most frequent words (ids 0..15), whose columns would
@@ -244,8 +255,9 @@ int w2v_set_ordered_copies(int copies, int twins);
  *      raw Zipf stream;
  *   2  off: no shadow copies, every column is read and updated in place;
  *  -1  (default) decided per launch and per table on the device: no shadow copies for a table
- *      unless at least 1/16 of the word ids read from it are among those 16, or at least 1/48 are
- *      id 0 (neither holds after frequent-word subsampling; the second holds for negatives drawn
+ *      unless at least 1/16 of the word ids read from it are occurrences of the launch's 16 most
+ *      frequent words, or at least 1/48 of its most frequent word (neither holds after
+ *      frequent-word subsampling; the second holds for negatives drawn
  *      with the reference's closed form, Word2Vec.scala:349-358); otherwise combining for launches
  *      with at least 2048 wavefronts in flight, where that many updates are invisible to each
  *      other anyway, and exact for smaller ones. */

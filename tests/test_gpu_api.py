@@ -80,7 +80,8 @@ def test_async_calls_timers_and_stream(lib, oracle):
     WAd, WBd = torch.from_numpy(WA).cuda(), torch.from_numpy(WB).cuda()
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()                       # default priority
-    assert lib.w2v_get_stream() is None
+    own = lib.w2v_get_stream()                         # the calling thread's own launch stream
+    assert own is not None and own != stream.cuda_stream
     try:
         assert lib.w2v_set_stream(stream.cuda_stream) == 0
         assert lib.w2v_get_stream() == stream.cuda_stream
@@ -91,8 +92,11 @@ def test_async_calls_timers_and_stream(lib, oracle):
         ms = t.elapsed_ms()
         synchronize()
         assert 0.0 < ms < 1000.0
+        assert lib.w2v_set_stream(None) == 0           # the legacy default stream, explicitly
+        assert lib.w2v_get_stream() is None
     finally:
-        lib.w2v_set_stream(None)
+        lib.w2v_reset_stream()
+    assert lib.w2v_get_stream() == own
     Ao, Bo = A.copy(), B.copy()
     oracle.word2vecNeg(d, G, 5, 5, WA, WB, Ao, Bo, 0.01, 0.0, 1)
     assert np.abs(Ad.cpu().numpy() - Ao).max() <= 1e-4
@@ -118,19 +122,25 @@ def test_two_host_threads_call_concurrently(lib, oracle):
 
     def work(j):
         dv = j["dev"]
+        j["stream"] = lib.w2v_get_stream()
         for _ in range(5):
             j["err"].append(CUMACH.word2vecPos(d, j["W"].shape[0], skip, dv["W"], dv["LB"],
                                                dv["UB"], dv["A"], dv["B"], 0.01, 0.5))
         j["err"].append(CUMACH.word2vecEvalPosF64(d, j["W"].shape[0], skip, dv["W"], dv["LB"],
                                                   dv["UB"], dv["A"], dv["B"], j["ret"]))
+        j["err"].append(lib.w2v_release_thread())      # the thread ends: scratch and stream back
 
     threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
     for t in threads:
         t.start()
     for t in threads:
         t.join()
+    # each thread launched on a stream of its own (the reference library's per-thread default
+    # stream, jni/src/configure:158,196): neither the other thread's nor this thread's
+    streams = {j["stream"] for j in jobs} | {lib.w2v_get_stream()}
+    assert None not in streams and len(streams) == 3
     for j in jobs:
-        assert j["err"] == [0] * 6
+        assert j["err"] == [0] * 7
         Ao, Bo = j["A"].copy(), j["B"].copy()
         for _ in range(5):
             oracle.word2vecPos(d, j["W"].shape[0], skip, j["W"], j["LB"], j["UB"], Ao, Bo, 0.01,

@@ -1,0 +1,225 @@
+"""The bfloat16-storage update operators at the full shape of their configuration (vocab 3M,
+Zipf(1.1), 1M-token launches) and on a raw Zipf(1.1) stream (needs an MI355X).
+
+First-order sums.  One launch with one table at zero and a step so small that every dot product
+stays ~0: g is then +-lr/2 for every pair and the zero table ends, to first order, as
+(lr/2) * (sum of its partners' columns), whatever the order of the updates
+(jni/src/BIDMach_CPUMACH.c:57-61, :239-254 of the reference, with sigmoid(0) = 1/2).  A
+contribution that is lost or applied twice shows in its row.  What the bfloat16 tables add is the
+stochastic rounding of every write-back: it is unbiased, so the share of all contributions that
+is missing must still be ~0, but a row that received k updates carries a random error of about
+2^-8 * sqrt(k) / 3 of its value (words among the first 1024, which go through fp32 side buffers,
+are rounded once).  Rows are therefore checked where a lost update would stand out, at up to 8
+contributions (a lost one is 12 % or more of the row, rounding 1 %), and all rows through the
+missing share.
+
+Held-out loss.  The configuration's own distribution (Zipf 1.1: 15 % of the tokens are word 0) on
+a raw stream, at a size the single-threaded bfloat16 oracle can afford: vocab 10k, dim 100, 30
+minibatches of 100k tokens, default settings (the launches are full of frequent words, so the
+ordered bfloat16 kernels run), against the sequential bfloat16 oracle.
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from bidmach_amd import corpus
+from oracle import cpumach
+
+pytestmark = pytest.mark.gpu
+
+V, D, N, SKIP, NNEG, NREUSE, ZIPF = 3_000_000, 32, 1_000_000, 5, 5, 5, 1.1
+LR = 1.0e-9
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from bidmach_amd.cumach import CUMACH, load_library
+    load_library()
+    return torch, CUMACH
+
+
+def dev(torch, x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def dev16(torch, h):
+    return torch.from_numpy(np.ascontiguousarray(h).view(np.int16)).cuda()
+
+
+def launch(wsample):
+    zc = corpus.zipf_cdf(V, ZIPF)
+    nc = corpus.unigram_pow_cdf(V, ZIPF, 0.75)
+    W = corpus.zipf_stream(N, V, ZIPF, seed=4321, cdf=zc)
+    rng = np.random.Generator(np.random.PCG64(17))
+    if wsample > 0:
+        W = corpus.subsample(W, V, wsample, rng)
+    LB, UB = corpus.window_bounds(N, SKIP, rng)
+    WA, WB, G = corpus.negative_groups(W, LB, UB, NNEG, NREUSE, rng, neg_cdf=nc)
+    return W, LB, UB, WA, WB, G
+
+
+def pos_pairs(W, LB, UB):
+    idx = np.arange(N, dtype=np.int64)
+    cs, xs = [], []
+    for j in range(-SKIP, SKIP + 1):
+        if j == 0:
+            continue
+        p = idx + j
+        ok = (W >= 0) & (LB <= j) & (j <= UB) & (p >= 0) & (p < N)
+        ok[ok] &= W[p[ok]] >= 0
+        cs.append(W[idx[ok]])
+        xs.append(W[p[ok]])
+    return np.concatenate(cs), np.concatenate(xs)
+
+
+def neg_pairs(WA, WB, G):
+    wa = np.repeat(WA.reshape(G, NNEG), NREUSE, axis=1).reshape(-1)
+    wb = np.tile(WB.reshape(G, NREUSE), (1, NNEG)).reshape(-1)
+    return wa, wb
+
+
+def partner_sums(rows, cols, T):
+    """(sum over the pairs of T[cols[p]] per row word, in float64; contributions per row word)."""
+    M = sp.coo_matrix((np.ones(rows.shape[0]), (rows, cols)), shape=(V, V)).tocsr()
+    return M @ T.astype(np.float64), np.asarray(M.sum(1)).ravel()
+
+
+def check(got, want, count, what):
+    norm = np.sqrt((want * want).sum(1))
+    touched = count > 0
+    err = np.sqrt(((got - want) ** 2).sum(1))
+    rel = np.zeros_like(err)
+    ok = norm > 0
+    rel[ok] = err[ok] / norm[ok]
+    missing = ((want - got) * want).sum() / (want * want).sum()
+    few = touched & (count <= 8)
+    bad = int((rel[few] > 0.05).sum())
+    print("\n%s: %d rows touched, %d of them with at most 8 contributions, of which beyond 5 %%: "
+          "%d; largest row error %.3f; missing share of all contributions %+.2e"
+          % (what, int(touched.sum()), int(few.sum()), bad, rel.max(), missing))
+    assert np.all(got[~touched] == 0.0), what + ": a row nobody touched changed"
+    assert few.sum() > 1000
+    assert bad == 0, what                   # no row lost (or doubled) one of its few updates
+    assert abs(missing) <= 1e-3, what       # and the sum of all rows is unbiased
+
+
+@pytest.mark.parametrize("wsample", [0.0, 1.0e-4], ids=["raw", "subsampled"])
+def test_bf16_full_shape_first_order_sums(gpu, wsample):
+    torch, CUMACH = gpu
+    rng = np.random.default_rng(3)
+    T16 = cpumach.bf16_truncate((rng.standard_normal((V, D)) * 0.2).astype(np.float32))
+    T = cpumach.bf16_widen(T16)
+    Z16 = np.zeros((V, D), np.uint16)
+    W, LB, UB, WA, WB, G = launch(wsample)
+    dW, dLB, dUB, dWA, dWB = (dev(torch, x) for x in (W, LB, UB, WA, WB))
+    pc, px = pos_pairs(W, LB, UB)
+    na, nb = neg_pairs(WA, WB, G)
+    tag = "bf16 tables, vocab 3M, Zipf(1.1), %s" % ("raw" if wsample == 0 else "subsampled")
+
+    def run(op, zero_is_a, seed):
+        A = dev16(torch, Z16 if zero_is_a else T16)
+        B = dev16(torch, T16 if zero_is_a else Z16)
+        if op == "pos":
+            err = CUMACH.word2vecPosBf16(D, N, SKIP, dW, dLB, dUB, A, B, LR, 0.0, seed)
+        else:
+            err = CUMACH.word2vecNegBf16(D, G, NNEG, NREUSE, dWA, dWB, A, B, LR, 0.0, seed)
+        assert err == 0
+        other = (B if zero_is_a else A).cpu().numpy().view(np.uint16)
+        assert np.array_equal(other, T16)   # a step of 1e-9 never moves the random table's bits
+        return cpumach.bf16_widen((A if zero_is_a else B).cpu().numpy().view(np.uint16))
+
+    want, cnt = partner_sums(pc, px, T)
+    check(run("pos", True, 1), 0.5 * LR * want, cnt, tag + ", pos, A table")
+    want, cnt = partner_sums(px, pc, T)
+    check(run("pos", False, 2), 0.5 * LR * want, cnt, tag + ", pos, B table")
+    want, cnt = partner_sums(na, nb, T)
+    check(run("neg", True, 3), -0.5 * LR * want, cnt, tag + ", neg, A table")
+    want, cnt = partner_sums(nb, na, T)
+    check(run("neg", False, 4), -0.5 * LR * want, cnt, tag + ", neg, B table")
+
+
+def test_bf16_raw_zipf11_stream_heldout_loss(gpu, oracle):
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import f32_to_bf16, load_library
+    lib = load_library()
+    assert lib.w2v_get_ordered_mode() == -1
+    hot = lib.w2v_get_bf16_hot_words()
+    Vs, Ds, Ns, K, LR0 = 10000, 100, 100000, 30, 0.025
+    zc = corpus.zipf_cdf(Vs, ZIPF)
+    nc = corpus.unigram_pow_cdf(Vs, ZIPF, 0.75)
+
+    def mb(i):
+        W = corpus.zipf_stream(Ns, Vs, ZIPF, seed=1234 + i, cdf=zc)
+        rng = np.random.Generator(np.random.PCG64(99 + i))
+        LB, UB = corpus.window_bounds(Ns, SKIP, rng)
+        WA, WB, G = corpus.negative_groups(W, LB, UB, NNEG, NREUSE, rng, neg_cdf=nc)
+        return W, LB, UB, WA, WB, G
+
+    def lr(i):
+        return max(LR0 * (1.0 - i / K), LR0 * 1e-4)
+
+    def score(epos, eneg, G):
+        return -(epos + eneg / NNEG) / (G * NREUSE)
+
+    mbs = [mb(i) for i in range(K + 1)]
+
+    def cpu32(nt):
+        B, A = corpus.init_tables(Vs, Ds, 42)
+        for i in range(K):
+            W, LB, UB, WA, WB, G = mbs[i]
+            oracle.word2vecPos(Ds, Ns, SKIP, W, LB, UB, A, B, lr(i), 0.0, nt)
+            oracle.word2vecNeg(Ds, G, NNEG, NREUSE, WA, WB, A, B, lr(i) / NNEG, 0.0, nt)
+        W, LB, UB, WA, WB, G = mbs[K]
+        return score(oracle.word2vecEvalPos(Ds, Ns, SKIP, W, LB, UB, A, B, 8),
+                     oracle.word2vecEvalNeg(Ds, G, NNEG, NREUSE, WA, WB, A, B, 8), G)
+
+    def cpu16():
+        B, A = corpus.init_tables(Vs, Ds, 42)
+        A16, B16 = cpumach.bf16_truncate(A), cpumach.bf16_truncate(B)
+        for i in range(K):
+            W, LB, UB, WA, WB, G = mbs[i]
+            oracle.word2vecPosBf16(Ds, Ns, SKIP, W, LB, UB, A16, B16, lr(i), 0.0, 2 * i, hot)
+            oracle.word2vecNegBf16(Ds, G, NNEG, NREUSE, WA, WB, A16, B16, lr(i) / NNEG, 0.0,
+                                   2 * i + 1, hot)
+        W, LB, UB, WA, WB, G = mbs[K]
+        return score(oracle.word2vecEvalPosBf16(Ds, Ns, SKIP, W, LB, UB, A16, B16),
+                     oracle.word2vecEvalNegBf16(Ds, G, NNEG, NREUSE, WA, WB, A16, B16), G)
+
+    def gpu16():
+        Bh, Ah = corpus.init_tables(Vs, Ds, 42)
+        A = torch.zeros(Vs * Ds, dtype=torch.int16, device="cuda")
+        B = torch.zeros(Vs * Ds, dtype=torch.int16, device="cuda")
+        f32_to_bf16(Vs * Ds, dev(torch, Ah), A)
+        f32_to_bf16(Vs * Ds, dev(torch, Bh), B)
+        for i in range(K):
+            W, LB, UB, WA, WB, G = mbs[i]
+            assert CUMACH.word2vecPosBf16(Ds, Ns, SKIP, dev(torch, W), dev(torch, LB),
+                                          dev(torch, UB), A, B, lr(i), 0.0, 2 * i) == 0
+            assert CUMACH.word2vecNegBf16(Ds, G, NNEG, NREUSE, dev(torch, WA), dev(torch, WB), A, B,
+                                          lr(i) / NNEG, 0.0, 2 * i + 1) == 0
+        W, LB, UB, WA, WB, G = mbs[K]
+        ret = torch.zeros(2, dtype=torch.float64, device="cuda")
+        assert CUMACH.word2vecEvalPosBf16(Ds, Ns, SKIP, dev(torch, W), dev(torch, LB),
+                                          dev(torch, UB), A, B, ret[0:1]) == 0
+        assert CUMACH.word2vecEvalNegBf16(Ds, G, NNEG, NREUSE, dev(torch, WA), dev(torch, WB), A, B,
+                                          ret[1:2]) == 0
+        r = ret.cpu().numpy()
+        return score(float(r[0]), float(r[1]), G)
+
+    seq32 = cpu32(1)
+    par32 = {t: cpu32(t) for t in (4, 8, 16)}
+    band = max(abs(v / seq32 - 1.0) for v in par32.values()) + 0.005
+    seq16 = cpu16()
+    got = [gpu16(), gpu16()]
+    print("\nraw Zipf(1.1), vocab 10k, 30 minibatches: fp32 oracle 1 thread %.5f (%s; band %.2f%%); "
+          "bfloat16 oracle 1 thread %.5f (%+.2f%% of the fp32 one); gpu bfloat16, default "
+          "settings, two runs: %s"
+          % (seq32, ", ".join("T=%d %+.2f%%" % (t, 100.0 * (v / seq32 - 1.0))
+                              for t, v in par32.items()), 100.0 * band, seq16,
+             100.0 * (seq16 / seq32 - 1.0),
+             ", ".join("%.5f (%+.2f%%)" % (g, 100.0 * (g / seq16 - 1.0)) for g in got)))
+    assert 0.005 <= band <= 0.10
+    for g in got:
+        assert np.isfinite(g) and abs(g / seq16 - 1.0) <= band, (g, seq16, band)

@@ -7,10 +7,11 @@ oracle check at its own size (needs an MI355X; about two minutes of host time).
       forward operators on the oracle-trained tables within 1e-5; (b) on the raw stream, where
       the ordered kernels run (with their 16-A-column instance) and where at lr 0.025 the oracle
       itself ends at seven times the untrained loss: the device must fail the same way, within
-      5 % (the oracle's 8- and 16-thread runs are 1 % apart; the device lands 2-3.5 % above).
+      the band the oracle's own runs span (two 16-thread runs against its 8-thread run) + 0.5 %.
   bfloat16 tables, vocab 3M, dim 300, 1M-token minibatch of a Zipf(1.1) stream:
       the forward operators against the bfloat16 oracle (1e-5) on tables that one full-size
-      update call has gone over, and that update call against a first-order sum.
+      update call has gone over.  (That update call itself is checked against first-order sums,
+      and the raw Zipf(1.1) loss against the bfloat16 oracle, in tests/test_gpu_bf16_full_size.py.)
 """
 import numpy as np
 import pytest
@@ -98,14 +99,18 @@ def test_dim512_window10_neg15_full_shape(oracle):
             # 1.386), and where it ends moves by several percent from one multi-threaded run of
             # the oracle to the next (16 threads: 9.98 to 10.41 seen).  The run with fewer threads
             # is the one nearer to the sequential order: the device is compared with an 8-thread
-            # run, within the distance of the 16-thread run from it plus 5 %.
+            # run, within what two 16-thread runs of the oracle itself use up, plus 0.5 %.
             assert ref > 5.0
             ref8 = heldout(*cpu_train(8))[0]
-            band = abs(ref / ref8 - 1.0) + 0.05
-            print("raw stream: the oracle on 8 threads %.5f (16 threads %+.2f%%, gpu %+.2f%%); "
-                  "band %.1f%%" % (ref8, 100.0 * (ref / ref8 - 1.0), 100.0 * (got / ref8 - 1.0),
-                                   100.0 * band))
-            assert band <= 0.25, band
+            ref16b = heldout(*cpu_train(16))[0]
+            # (two runs can happen to agree: the spread is taken to be 1.5 % at least, the smallest
+            # seen between an 8- and a 16-thread run here)
+            band = max(abs(ref / ref8 - 1.0), abs(ref16b / ref8 - 1.0), 0.015) + 0.005
+            print("raw stream: the oracle on 8 threads %.5f (16 threads %+.2f%% and %+.2f%%, gpu "
+                  "%+.2f%%); band %.1f%%"
+                  % (ref8, 100.0 * (ref / ref8 - 1.0), 100.0 * (ref16b / ref8 - 1.0),
+                     100.0 * (got / ref8 - 1.0), 100.0 * band))
+            assert band <= 0.10, band
             assert abs(got / ref8 - 1.0) <= band, (got, ref8, band)
 
 

@@ -142,10 +142,10 @@ def test_a_word_twice_among_a_groups_b_words_sees_its_first_update(gpu, oracle):
     assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
 
 
-def test_launches_without_frequent_words_keep_the_throughput_kernels(gpu, oracle):
-    """The decision is made on the device from the ids of the launch: with no id below 16 the
-    ordered kernels return at once, whatever the collisions (here: the same heavy collisions on
-    ids 100..105, where the tile's snapshot semantics show)."""
+def test_the_decision_does_not_depend_on_how_the_vocabulary_is_numbered(gpu, oracle):
+    """The decision is made on the device from how often the words of the launch occur, not from
+    their ids: the same heavy collisions on ids 100..105 (no id below 16) take the ordered form
+    by default and reproduce the sequential result."""
     rng = np.random.default_rng(5)
     d, skip = 100, 5
     A, B, W, LB, UB = tiny_colliding(rng, d, 6, 60, skip)
@@ -156,7 +156,90 @@ def test_launches_without_frequent_words_keep_the_throughput_kernels(gpu, oracle
     Ao, Bo = A2.copy(), B2.copy()
     oracle.word2vecPos(d, 60, skip, W2, LB, UB, Ao, Bo, 0.05, 0.0, 1)
     Ag, Bg = parity.gpu_pos(gpu, d, skip, W2, LB, UB, A2, B2, 0.05, 0.0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
+    G, nwa, nwb = 16, 3, 3
+    WA = np.concatenate([100 + rng.permutation(6)[:nwa] for _ in range(G)]).astype(np.int32)
+    WB = np.concatenate([100 + rng.permutation(6)[:nwb] for _ in range(G)]).astype(np.int32)
+    Ao, Bo = A2.copy(), B2.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.05, 0.0, 1)
+    Ag, Bg = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A2, B2, 0.05, 0.0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
+
+
+def test_launches_without_frequent_words_keep_the_throughput_kernels(gpu, oracle):
+    """2000 tokens, every word once: no word is frequent, so the default is the tiled kernel,
+    whose tiles of 16 adjacent tokens work from one snapshot of their columns: at a large step its
+    result is visibly not the sequential one (adjacent windows share their context positions),
+    while the ordered form, forced onto one worker, is."""
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(6)
+    d, skip, n = 100, 5, 2000
+    A = (rng.standard_normal((n, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((n, d)) * 0.3).astype(np.float32)
+    W = rng.permutation(n).astype(np.int32)
+    LB, UB = corpus.window_bounds(n, skip, rng)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecPos(d, n, skip, W, LB, UB, Ao, Bo, 0.3, 0.0, 1)
+    Ag, Bg = parity.gpu_pos(gpu, d, skip, W, LB, UB, A, B, 0.3, 0.0)
     assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) > 1e-3
+    lib.w2v_set_ordered_mode(1)
+    lib.w2v_set_ordered_workers(1, 1)       # one worker: the sequential order itself
+    try:
+        Ag, Bg = parity.gpu_pos(gpu, d, skip, W, LB, UB, A, B, 0.3, 0.0)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+        lib.w2v_set_ordered_workers(0, 0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
+
+
+def test_a_b_word_of_two_tiles_of_a_wide_group_sees_its_first_update(gpu, oracle):
+    """Groups with more than 8 B words pass their B columns through registers in tiles of 8; a
+    word that is a B word in two tiles is read for the second one as the first one's adds left it
+    (BIDMach_CPUMACH.c:219-246 walks the rows one after the other).  The ids are spread over a
+    large vocabulary so that no word of the launch is frequent and the throughput kernel runs."""
+    rng = np.random.default_rng(12)
+    d, V, G, nwa, nwb = 100, 40000, 300, 4, 10
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    ids = rng.permutation(V)[:G * (nwa + nwb)].astype(np.int32)
+    WA = ids[:G * nwa].copy()
+    WB = ids[G * nwa:].copy()
+    WB[8::nwb] = WB[0::nwb]          # row 8 (second tile) repeats row 0 (first tile)
+    WB[9::nwb] = WB[5::nwb]          # and row 9 repeats row 5
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecNeg(d, G, nwa, nwb, WA, WB, Ao, Bo, 0.05, 0.0, 1)
+    Ag, Bg = parity.gpu_neg(gpu, d, G, nwa, nwb, WA, WB, A, B, 0.05, 0.0)
+    assert max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max()) <= 2e-5
+
+
+def test_ordered_launch_of_a_shape_without_a_row_by_row_instance(gpu, oracle):
+    """17 A words per group fit no instance of the row-by-row kernel: an ordered launch then runs
+    the group-at-a-time kernels on a few workgroups, for the single-table, the wide and the sliced
+    operator alike.  On colliding words that order is not the sequential one, so the check is the
+    collision-free parity with the ordered form forced."""
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    lib.w2v_set_ordered_mode(1)
+    try:
+        parity.test_neg_update_matches_oracle(gpu, oracle, 0.5, 200, 17, 5, 60)
+        parity.test_neg_update_matches_oracle(gpu, oracle, 0.5, 200, 17, 12, 60)
+        islice, nslices, nhead, maxcols, dohead, dual = sliced_slicings()[1]
+        sliced_mod().test_neg_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols,
+                                                   dohead, dual, 200, 17, 5, 0.5)
+        sliced_mod().test_neg_slice_matches_oracle(gpu, oracle, islice, nslices, nhead, maxcols,
+                                                   dohead, dual, 200, 17, 12, 0.5)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+
+
+def sliced_mod():
+    from tests import test_gpu_slice
+    return test_gpu_slice
+
+
+def sliced_slicings():
+    return sliced_mod().SLICINGS
 
 
 # ---- sliced, multi-part models (word2vecPosSlice / word2vecNegSlice) ---------------------------
