@@ -17,12 +17,15 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_NAME = "libbidmachhip-linux-x86_64.so"
 LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
 # The name the reference's Java side asks its loader for (CUMACH.java:9 loads "bidmachcuda";
-# artefact libbidmachcuda-linux-x86_64.so, jni/src/Makefile:20-21): a link to the library, so a
-# BIDMach installation finds it under the name it already uses.
+# artefact libbidmachcuda-linux-x86_64.so, jni/src/Makefile:20-21): a link to the JNI glue where a
+# JDK let jni/Makefile build it (the glue is linked against the HIP library), else to the HIP
+# library itself, so a BIDMach installation finds the operators under the name it already uses.
 ALIAS_NAME = "libbidmachcuda-linux-x86_64.so"
 ALIAS_PATH = os.path.join(LIB_DIR, ALIAS_NAME)
+JNI_NAME = "libbidmachcuda-jni-linux-x86_64.so"
+JNI_PATH = os.path.join(LIB_DIR, JNI_NAME)
 
-SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_neg_wide.hip", "w2v_neg_rows.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
+SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_neg_wide.hip", "w2v_neg_rows.hip", "w2v_any_shape.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
            "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_bf16_neg_rows.hip", "w2v_bf16_neg_rows_unaligned.hip", "w2v_api.hip"]
 
 HIPCC_FLAGS = [
@@ -65,12 +68,25 @@ def build(extra_flags=(), verbose=True, out=None):
     if verbose:
         print("built", out)
     if out == LIB_PATH:
-        if os.path.lexists(ALIAS_PATH):
-            os.remove(ALIAS_PATH)
-        os.symlink(LIB_NAME, ALIAS_PATH)
-        # where a JDK is installed the JNI glue takes the alias's place (jni/Makefile)
-        subprocess.check_call(["make", "-s", "-C", os.path.join(os.path.dirname(HERE), "jni")])
+        link_alias(build_jni_glue())
     return out
+
+
+def build_jni_glue():
+    """Runs jni/Makefile (it builds only where it finds jni.h).  True if the glue library is there
+    afterwards.  A missing `make` or a failed glue build does not fail the HIP build."""
+    try:
+        subprocess.check_call(["make", "-s", "-C", os.path.join(os.path.dirname(HERE), "jni")])
+    except (OSError, subprocess.CalledProcessError) as e:
+        sys.stderr.write("JNI glue not built: %s\n" % e)
+        return False
+    return os.path.isfile(JNI_PATH)
+
+
+def link_alias(to_jni):
+    if os.path.lexists(ALIAS_PATH):
+        os.remove(ALIAS_PATH)
+    os.symlink(JNI_NAME if to_jni else LIB_NAME, ALIAS_PATH)
 
 
 if __name__ == "__main__":

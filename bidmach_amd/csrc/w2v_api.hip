@@ -166,8 +166,17 @@ hipError_t shadow_buffers(w2v::Shadow* out) {
   return hipSuccess;
 }
 
-bool bad_common(int nrows, int ncols) {
-  return nrows <= 0 || nrows > w2v::max_rows() || ncols < 0;
+// any_rows: the operator has a kernel for columns of any length (w2v_any_shape.hip)
+bool bad_common(int nrows, int ncols, bool any_rows = false) {
+  return nrows <= 0 || (!any_rows && nrows > w2v::max_rows()) || ncols < 0;
+}
+
+// Whether a negative-pass shape goes to the any-shape kernels: columns longer than a wave holds
+// in registers, more B words than a wave has lanes, or a wide group whose A columns do not fit
+// in LDS.
+bool neg_needs_any(int nrows, int nwa, int nwb) {
+  return nrows > w2v::max_rows() || nwb > w2v::max_nwb() ||
+         (nwb > 8 && !w2v::neg_wide_fits(nrows, nwa));
 }
 
 int finish(hipError_t launch_err, bool sync) {
@@ -182,9 +191,12 @@ int finish(hipError_t launch_err, bool sync) {
 
 int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A, float* B,
              float lrate, float vexp, bool sync) {
-  if (bad_common(nrows, ncols)) return (int)hipErrorInvalidValue;
+  if (bad_common(nrows, ncols, true)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
+  if (nrows > w2v::max_rows())
+    return finish(w2v::launch_pos_any(launch_stream(), nrows, ncols, W, LB, UB, A, B, lrate, vexp),
+                  sync);
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
@@ -195,10 +207,16 @@ int pos_impl(int nrows, int ncols, int shift, int* W, int* LB, int* UB, float* A
 
 int neg_impl(int nrows, int ncols, int idlimit, int nwa, int nwb, int* WA, int* WB, float* A,
              float* B, float lrate, float vexp, bool sync) {
-  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || idlimit < 0)
+  if (bad_common(nrows, ncols, true) || nwa < 0 || nwb < 0 || idlimit < 0)
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
+  if (neg_needs_any(nrows, nwa, nwb)) {
+    if (!w2v::neg_any_fits(nwa, nwb)) return (int)hipErrorInvalidValue;
+    return finish(w2v::launch_neg_any(launch_stream(), nrows, ncols, idlimit, nwa, nwb, WA, WB, A,
+                                      B, lrate, vexp),
+                  sync);
+  }
   w2v::Shadow shadow{};
   hipError_t err = shadow_buffers(&shadow);
   if (err != hipSuccess) return (int)err;
@@ -209,12 +227,16 @@ int neg_impl(int nrows, int ncols, int idlimit, int nwa, int nwb, int* WA, int* 
 
 int eval_pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, float* B, float* r32,
                   double* r64, bool sync) {
-  if (bad_common(nrows, ncols) || (!r32 && !r64)) return (int)hipErrorInvalidValue;
+  if (bad_common(nrows, ncols, true) || (!r32 && !r64)) return (int)hipErrorInvalidValue;
   if (ncols == 0) return 0;
   if (!W || !LB || !UB || !A || !B) return (int)hipErrorInvalidValue;
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
   if (err != hipSuccess) return (int)err;
+  if (nrows > w2v::max_rows())
+    return finish(w2v::launch_eval_pos_any(launch_stream(), nrows, ncols, W, LB, UB, A, B,
+                                           g_eval_floor.load(), partials, r32, r64),
+                  sync);
   return finish(w2v::launch_eval_pos(launch_stream(), nrows, ncols, W, LB, UB, A, B,
                                      g_eval_floor.load(), partials, r32, r64),
                 sync);
@@ -222,13 +244,19 @@ int eval_pos_impl(int nrows, int ncols, int* W, int* LB, int* UB, float* A, floa
 
 int eval_neg_impl(int nrows, int ncols, int nwa, int nwb, int* WA, int* WB, float* A, float* B,
                   float* r32, double* r64, bool sync) {
-  if (bad_common(nrows, ncols) || nwa < 0 || nwb < 0 || nwb > w2v::max_nwb() || (!r32 && !r64))
+  if (bad_common(nrows, ncols, true) || nwa < 0 || nwb < 0 || (!r32 && !r64))
     return (int)hipErrorInvalidValue;
   if (ncols == 0 || nwa == 0 || nwb == 0) return 0;
   if (!WA || !WB || !A || !B) return (int)hipErrorInvalidValue;
   double* partials = nullptr;
   hipError_t err = eval_scratch(w2v::eval_partials_needed(ncols), &partials);
   if (err != hipSuccess) return (int)err;
+  // (the forward kernels tile over the B words, so only long columns and more than 64 B words
+  // need the any-shape kernel)
+  if (nrows > w2v::max_rows() || nwb > w2v::max_nwb())
+    return finish(w2v::launch_eval_neg_any(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, A, B,
+                                           g_eval_floor.load(), partials, r32, r64, 0),
+                  sync);
   return finish(w2v::launch_eval_neg(launch_stream(), nrows, ncols, nwa, nwb, WA, WB, A, B,
                                      g_eval_floor.load(), partials, r32, r64),
                 sync);

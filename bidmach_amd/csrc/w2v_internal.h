@@ -193,7 +193,28 @@ hipError_t launch_slice_eval_neg(hipStream_t stream, int nrows, int ncols, int n
                                  const int* WA, const int* WB, const SliceMap& m, double floorv,
                                  double* partials, float* Retval32, double* Retval64);
 
-// Largest nrows / nwb the register-resident kernels take; beyond them the calls fail with
+// The operators for any shape (w2v_any_shape.hip): one wave per work unit, columns walked in
+// chunks, untuned.  Taken for nrows beyond max_rows(), nwb beyond max_nwb(), and wide groups whose
+// A columns do not fit in LDS (neg_wide_fits).  neg_any_fits: the group's nwa x nwb steps and one
+// chunk of A deltas fit in LDS (else the negative operators fail with hipErrorInvalidValue).
+bool neg_wide_fits(int nrows, int nwa);
+bool neg_any_fits(int nwa, int nwb);
+hipError_t launch_pos_any(hipStream_t stream, int nrows, int ncols, const int* W, const int* LB,
+                          const int* UB, float* A, float* B, float lrate, float vexp);
+hipError_t launch_eval_pos_any(hipStream_t stream, int nrows, int ncols, const int* W,
+                               const int* LB, const int* UB, const float* A, const float* B,
+                               double floorv, double* partials, float* Retval32,
+                               double* Retval64);
+hipError_t launch_neg_any(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
+                          const int* WA, const int* WB, float* A, float* B, float lrate,
+                          float vexp);
+hipError_t launch_eval_neg_any(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
+                               const int* WA, const int* WB, const float* A, const float* B,
+                               double floorv, double* partials, float* Retval32, double* Retval64,
+                               int64_t partials_capacity);
+
+// Largest nrows / nwb the register-resident kernels take; the single-table fp32 operators go to
+// the any-shape kernels beyond them, the sliced and bfloat16 operators fail with
 // hipErrorInvalidValue.
 int max_rows();
 int max_nwb();

@@ -241,6 +241,12 @@ hipError_t launch_wide(hipStream_t stream, int d, int ngroups, int idlimit, int 
 
 }  // namespace
 
+bool neg_wide_fits(int nrows, int nwa) {
+  const int rounds = (nrows + kWave - 1) / kWave;
+  const int R = rounds <= 2 ? 2 : rounds <= 5 ? 5 : rounds <= 8 ? 8 : rounds <= 12 ? 12 : kMaxRounds;
+  return rounds <= kMaxRounds && ((size_t)2 * nwa * R * kWave + nwa) * sizeof(float) <= kWideMaxLds;
+}
+
 hipError_t launch_neg_wide(hipStream_t stream, int nrows, int ncols, int idlimit, int nwa, int nwb,
                            const int* WA, const int* WB, float* A, float* B, float lrate,
                            float vexp, const Shadow& shadow) {

@@ -836,71 +836,98 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
 // largest bin larger, and the words that are not frequent add about four ids to every bin, 0.4 %
 // of the sample over the kHeavyTop bins: both err towards "frequent".  One workgroup.
 constexpr int kHeavyThreads = 1024;
+constexpr int kHeavyWaves = kHeavyThreads / kWave;
 constexpr int kHeavySamples = 16384;
+constexpr int kHeavyPerThread = kHeavySamples / kHeavyThreads;
 constexpr int kHeavyBins = 4096;
+constexpr int kHeavyPerLane = kHeavyBins / kHeavyThreads;   // bins a lane looks after
 constexpr int kHeavyTop = kHotWords;
+static_assert(kHeavyWaves * kHeavyTop == kWave * kHeavyPerLane, "second stage: one wave, same shape");
+
+// The kHeavyTop largest of the kWave * kHeavyPerLane values a wave holds (v[k] of every lane),
+// largest first: out[r] is valid in every lane.  Wave-level only: no barrier.
+__device__ __forceinline__ void wave_top(int (&v)[kHeavyPerLane], int (&out)[kHeavyTop]) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int r = 0; r < kHeavyTop; ++r) {
+    int best = -1, at = 0;
+#pragma unroll
+    for (int k = 0; k < kHeavyPerLane; ++k) {
+      if (v[k] > best) {
+        best = v[k];
+        at = k;
+      }
+    }
+    int wbest = best, wlane = lane;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      const int ov = __shfl_xor(wbest, m, kWave), ol = __shfl_xor(wlane, m, kWave);
+      if (ov > wbest || (ov == wbest && ol < wlane)) {
+        wbest = ov;
+        wlane = ol;
+      }
+    }
+    out[r] = wbest;
+    if (lane == wlane) {
+#pragma unroll
+      for (int k = 0; k < kHeavyPerLane; ++k)
+        if (k == at) v[k] = -1;
+    }
+  }
+}
+
 __global__ void __launch_bounds__(kHeavyThreads)
 count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict__ ids2, int64_t n2,
                    int* __restrict__ out) {
   __shared__ int s_bins[kHeavyBins];
-  __shared__ int s_val[kHeavyThreads / kWave], s_idx[kHeavyThreads / kWave];
-  __shared__ int s_pick;
+  __shared__ int s_cand[kHeavyWaves * kHeavyTop];
+  __shared__ long long s_result[2];
   const int tid = threadIdx.x;
   for (int which = 0; which < 2; ++which) {
     const int* const p = which ? ids2 : ids;
     const int64_t len = which ? n2 : n;
-    long long top_sum = 0, top_one = 0;
+    if (tid < 2) s_result[tid] = 0;
     if (p != nullptr && len > 0) {
       for (int k = tid; k < kHeavyBins; k += kHeavyThreads) s_bins[k] = 0;
       __syncthreads();
       const int64_t stride = (len + kHeavySamples - 1) / kHeavySamples;
       const int64_t nsamp = (len + stride - 1) / stride;
-      for (int64_t k = tid; k < nsamp; k += kHeavyThreads) {
-        const int w = p[k * stride];
-        if (w >= 0) atomicAdd(&s_bins[((unsigned)w * 2654435761u) >> 20], 1);
+      int w[kHeavyPerThread];
+#pragma unroll
+      for (int k = 0; k < kHeavyPerThread; ++k) {   // all loads in flight together
+        const int64_t at = (int64_t)k * kHeavyThreads + tid;
+        w[k] = at < nsamp ? p[at * stride] : -1;
+      }
+#pragma unroll
+      for (int k = 0; k < kHeavyPerThread; ++k)
+        if (w[k] >= 0) atomicAdd(&s_bins[((unsigned)w[k] * 2654435761u) >> 20], 1);
+      __syncthreads();
+      // every wave picks the largest of its 256 bins, then the first wave the largest of those
+      int v[kHeavyPerLane], top[kHeavyTop];
+#pragma unroll
+      for (int k = 0; k < kHeavyPerLane; ++k) v[k] = s_bins[k * kHeavyThreads + tid];
+      wave_top(v, top);
+      if ((tid & 63) == 0) {
+#pragma unroll
+        for (int r = 0; r < kHeavyTop; ++r) s_cand[(tid >> 6) * kHeavyTop + r] = top[r];
       }
       __syncthreads();
-      for (int round = 0; round < kHeavyTop; ++round) {
-        int best = -1, at = 0;
-        for (int k = tid; k < kHeavyBins; k += kHeavyThreads) {
-          const int v = s_bins[k];
-          if (v > best) {
-            best = v;
-            at = k;
-          }
-        }
+      if (tid < kWave) {
 #pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) {
-          const int ov = __shfl_xor(best, m, kWave), oi = __shfl_xor(at, m, kWave);
-          if (ov > best || (ov == best && oi < at)) {
-            best = ov;
-            at = oi;
-          }
-        }
-        if ((tid & 63) == 0) {
-          s_val[tid >> 6] = best;
-          s_idx[tid >> 6] = at;
-        }
-        __syncthreads();
+        for (int k = 0; k < kHeavyPerLane; ++k) v[k] = s_cand[k * kWave + tid];
+        wave_top(v, top);
         if (tid == 0) {
-          int bv = -1, bi = 0;
-          for (int k = 0; k < kHeavyThreads / kWave; ++k) {
-            if (s_val[k] > bv) {
-              bv = s_val[k];
-              bi = s_idx[k];
-            }
-          }
-          s_pick = bv;
-          s_bins[bi] = 0;
+          long long sum = 0;
+#pragma unroll
+          for (int r = 0; r < kHeavyTop; ++r) sum += top[r] > 0 ? top[r] : 0;
+          // sampled counts scaled up to the whole array (dropped words, id < 0, stay in the total)
+          s_result[0] = sum * len / nsamp;
+          s_result[1] = (long long)(top[0] > 0 ? top[0] : 0) * len / nsamp;
         }
-        __syncthreads();
-        top_sum += s_pick;
-        if (round == 0) top_one = s_pick;
       }
-      // sampled counts scaled up to the whole array (dropped words, id < 0, stay in the total)
-      top_sum = top_sum * len / nsamp;
-      top_one = top_one * len / nsamp;
     }
+    __syncthreads();
+    const long long top_sum = s_result[0], top_one = s_result[1];
     for (int k = tid; k < kHotCountSlots; k += kHeavyThreads) {
       out[(2 * which) * kHotCountSlots + k] = k == 0 ? (int)min(top_sum, (long long)0x7fffffff) : 0;
       out[(2 * which + 1) * kHotCountSlots + k] = k == 0 ? (int)min(top_one, (long long)0x7fffffff) : 0;

@@ -45,7 +45,7 @@ int word2vecPos(int nrows, int ncols, int shift, int *W, int *LB, int *UB, float
 
 /* Replaces word2vecNeg, MatKernel.hpp:79 / DNN127.cu:1423-1452; arithmetic of
  * BIDMach_CPUMACH.c:186-264.  ncols groups; group i pairs the nwa words WA[i*nwa + j] (columns of
- * A) with the nwb words WB[i*nwb + k] (columns of B).  nwb <= w2v_max_nwb(). */
+ * A) with the nwb words WB[i*nwb + k] (columns of B).  Any nwa and nwb (see w2v_max_nwb). */
 int word2vecNeg(int nrows, int ncols, int nwa, int nwb, int *WA, int *WB, float *A, float *B,
                 float lrate, float vexp);
 
@@ -280,7 +280,14 @@ int w2v_get_hot_update_mode(void);
 int w2v_set_rare_update_mode(int mode);
 int w2v_get_rare_update_mode(void);
 
-/* Limits of the kernels: largest nrows and largest nwb. */
+/* Limits of the tuned kernels: largest nrows (1280) and largest nwb (64).  The four single-table
+ * fp32 operators (and word2vecNegFilt, the ...F64, ...Async and ...NoAlloc forms) take any shape:
+ * beyond these limits, and for groups of more than 8 B words whose A columns do not fit on chip
+ * (about nwa * ceil(nrows/64) > 300), they run one untuned wave-per-unit kernel, as the
+ * reference's CPU path takes any nrows, nwa and nwb (BIDMach_CPUMACH.c:37,206,212); that
+ * kernel's only bound is nwa * (nwb + 256) <= 16384 for the update (hipErrorInvalidValue
+ * beyond).  The sliced and the bfloat16 operators fail with hipErrorInvalidValue beyond the
+ * limits. */
 int w2v_max_rows(void);
 int w2v_max_nwb(void);
 

@@ -78,3 +78,29 @@ def test_jni_glue_binds_the_reference_natives_to_declared_functions():
 
 def test_release_thread_without_scratch_is_a_no_op():
     assert cumach.load_library().w2v_release_thread() == 0
+
+
+def test_jni_makefile_rebuilds_the_glue_and_the_alias_follows_it(tmp_path):
+    """jni/Makefile builds the glue into a regular file of its own, so make's time-stamp test
+    works (a target that is a symbolic link to the HIP library would always look up to date), and
+    bidmach_amd/build.py points the reference's artefact name at the glue only where it exists.
+    Dry run against a JAVA_HOME that holds an (empty) include/jni.h: nothing is compiled."""
+    import shutil
+    import subprocess
+    if shutil.which("make") is None:
+        pytest.skip("no make")
+    from bidmach_amd import build
+    (tmp_path / "include").mkdir()
+    (tmp_path / "include" / "jni.h").write_text("")
+    out = subprocess.run(["make", "-n", "-C", os.path.join(ROOT, "jni"), "JAVA_HOME=%s" % tmp_path],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert out.returncode == 0, out.stdout
+    if not os.path.exists(build.JNI_PATH):
+        assert "cumach_w2v_jni.cpp" in out.stdout and build.JNI_NAME in out.stdout, out.stdout
+    assert build.JNI_NAME != build.ALIAS_NAME
+    none = subprocess.run(["make", "-n", "-C", os.path.join(ROOT, "jni"), "JAVA_HOME=/nonexistent"],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert none.returncode == 0 and "not built" in none.stdout
+    if os.path.lexists(build.ALIAS_PATH):
+        want = build.JNI_NAME if os.path.isfile(build.JNI_PATH) else build.LIB_NAME
+        assert os.readlink(build.ALIAS_PATH) == want

@@ -298,10 +298,9 @@ def test_empty_and_rejected_arguments(gpu):
     assert float(ret.item()) == 0.0
     # rejected shapes and null pointers: hipErrorInvalidValue (1), no launch, no abort
     assert CUMACH.word2vecPos(0, 4, 5, I, I, I, A, B, 0.1, 0.5) == 1
-    assert CUMACH.word2vecPos(1281, 4, 5, I, I, I, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecPos(d, -1, 5, I, I, I, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecPos(d, 4, 5, None, I, I, A, B, 0.1, 0.5) == 1
-    assert CUMACH.word2vecNeg(d, 1, 5, 65, I, I, A, B, 0.1, 0.5) == 1    # more B words than lanes
+    assert CUMACH.word2vecNeg(d, 1, 200, 100, I, I, A, B, 0.1, 0.5) == 1   # no kernel holds this group
     assert CUMACH.word2vecNeg(d, 1, 5, 5, I, None, A, B, 0.1, 0.5) == 1
     assert CUMACH.word2vecEvalPos(d, 4, 5, I, I, I, A, B, None) == 1
     assert CUMACH.word2vecEvalNeg(d, 1, 5, 5, I, I, A, None, ret) == 1
