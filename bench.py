@@ -11,7 +11,8 @@ before the timed region starts.  Prints ONE JSON line.
 Other workloads (--workload) are the remaining configurations at their full shapes: dim 512 with
 window 10 and 15 negatives, the small vocab-10k configuration, forward-only scoring (--mode eval),
 and bfloat16 tables at vocab 3M (word2vecPosBf16 + word2vecNegBf16; its CPU baseline is the
-single-threaded bf16 oracle on a 300k-token sample).
+fp32 oracle on all host threads on the widened tables, with the single-threaded bfloat16 oracle
+on a 300k-token sample beside it).
 """
 import argparse
 import json
@@ -35,7 +36,7 @@ HEADLINE = "sgns_v1m_d300_w5_neg5_fp32"
 MEASURED_TRAFFIC = {
     HEADLINE: {
         # the kernels the library takes for this raw stream by itself
-        "ordered": {"neg_kernel": 36.97e9, "pos_kernel": 17.29e9,
+        "ordered": {"neg_kernel": 32.81e9, "pos_kernel": 20.69e9,
                     "source": "profiles/sgns_v1m_d300_ordered_step_kernel_stats_and_hbm_traffic.md"},
         # --ordered-mode 0
         "throughput": {"neg_kernel": 29.35e9, "pos_kernel": 4.63e9,
@@ -397,13 +398,22 @@ class Leg:
         """The CPU baseline of this leg on `nmb` of its minibatches (bf16: a 300k-token sample on
         the single-threaded bf16 oracle)."""
         cfg = self.cfg
+        threads = host_threads()
         if self.bf16:
+            # the same arithmetic on fp32 tables (the bfloat16 tables widened), all host threads,
+            # is what a CPU would run; the bfloat16 oracle itself has one thread
+            wps32, dt32 = cpu_baseline(cfg, self.host_mbs[:1], self.lrate0,
+                                       self.lrate0 / cfg["nneg"], self.vexp, threads)
             wps, dt, m = cpu_baseline_bf16(cfg, self.host_mbs[0], self.lrate0,
                                            self.lrate0 / cfg["nneg"], self.vexp, 300_000)
-            return {"value": wps, "unit": "words/s", "cores": 1, "kind": "port",
-                    "sample": "the first %d tokens of one minibatch and their groups, pos+neg, "
-                              "single-threaded bf16 oracle, %.1f s wall" % (m, dt)}
-        threads = host_threads()
+            return {"value": wps32, "unit": "words/s", "cores": threads, "kind": "port",
+                    "sample": "one full minibatch (%d tokens) of the same workload on fp32 tables "
+                              "(the fp32 oracle: same arithmetic, no rounding of the write-back), "
+                              "pos+neg, %.1f s wall" % (cfg["tokens"], dt32),
+                    "bf16_oracle_one_thread": {
+                        "value": wps, "unit": "words/s", "cores": 1,
+                        "sample": "the first %d tokens of one minibatch and their groups, "
+                                  "pos+neg, %.1f s wall" % (m, dt)}}
         sample = self.host_mbs[:nmb]
         wps, dt = cpu_baseline(cfg, sample, self.lrate0, self.lrate0 / cfg["nneg"], self.vexp,
                                threads)

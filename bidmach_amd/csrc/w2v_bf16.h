@@ -248,6 +248,40 @@ __device__ __forceinline__ void add_col16(uint16_t* col, const float (&seen)[2 *
   }
 }
 
+// col[e] = narrow(seen[e] + delta[e]) for the lane's elements with plain device-scope stores: no
+// exchange, nothing to wait for.  What another wave added to the column between this wave's read
+// of `seen` and this store is overwritten, so this is for the words that are rare within a launch
+// of the ordered kernels (a few hundred workers, each between a column's read and its write for a
+// few microseconds: two updates of a word that occurs a handful of times practically never
+// overlap), and it is the closest this library gets to the atomic-free stochastic-rounded
+// write-back of bfloat16 tables.  Same random bits as the exchange: without an overlapping update
+// the stored bits are the same.
+template <int RP, bool ALIGNED>
+__device__ __forceinline__ void store_col16(uint16_t* col, const float (&seen)[2 * RP],
+                                            const float (&delta)[2 * RP], int lane, int d,
+                                            uint32_t key) {
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    const int e = r * 128 + 2 * lane;
+    if (e < d) {
+      const uint32_t lo = sr_narrow(seen[2 * r] + delta[2 * r], key, (uint32_t)e);
+      if (ALIGNED) {
+        // (an odd d is never ALIGNED, so e + 1 < d here)
+        const uint32_t hi = sr_narrow(seen[2 * r + 1] + delta[2 * r + 1], key, (uint32_t)(e + 1));
+        __hip_atomic_store(reinterpret_cast<uint32_t*>(col + e), lo | (hi << 16), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        __hip_atomic_store(col + e, (uint16_t)lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (e + 1 < d)
+          __hip_atomic_store(col + e + 1,
+                             (uint16_t)sr_narrow(seen[2 * r + 1] + delta[2 * r + 1], key,
+                                                 (uint32_t)(e + 1)),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+}
+
 // Frequent words.  Word ids are frequency ranks, so the first few hundred ids take most of the
 // updates of a call, and a compare-and-swap on a column that thousands of waves update at once
 // fails nearly every time.  The columns of the words below `n` therefore have an fp32 side

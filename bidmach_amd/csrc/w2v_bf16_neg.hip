@@ -224,6 +224,11 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
   hipError_t lerr = hipGetLastError();
   if (lerr != hipSuccess || EVAL) return lerr;
   if (rows) {
+    const int64_t chains = ordered_neg_chains(kWavesPerBlock, kNegRowWorkersBf16);
+    // words that are rare within the launch are written back with plain stores (store_col16)
+    lerr = prepare_rare_words(stream, WA, (int64_t)n * nwa, WB, (int64_t)n * nwb, 0x7fffffff, n,
+                              chains, &shadow, kRareCapOrderedBf16);
+    if (lerr != hipSuccess) return lerr;
     lerr = launch_neg_rows_bf16(stream, d, n, nwa, nwb, WA, WB, A, B, lrate, vexp, seed, hot,
                                 ordered_neg_chains(kWavesPerBlock, kNegRowWorkersBf16), shadow);
     if (lerr != hipSuccess) return lerr;

@@ -9,7 +9,9 @@
 // once (:244-246) - to the side buffer of a frequent word with float atomics, else into the table
 // by compare-and-swap with stochastic rounding - before the wave turns to the next B word; the A
 // columns are written after the last row (:248-254).  The next row's column is requested while
-// the current row is worked on; the exchanges of the A columns are in flight together.  (Keeping
+// the current row is worked on; the exchanges of the A columns are in flight together.  Words
+// that are rare within the launch (counted on the device beforehand) are written back with plain
+// stores instead of exchanges: nothing to wait for.  (Keeping
 // the rows' exchanges in flight as well costs more registers than a wave has: the results spill
 // and every spill waits for its exchange, 136 against 122 ms on a 1.2M-group launch.)
 // Sums are formed in the order of the group-at-a-time kernel (w2v_bf16_neg.hip) and every write
@@ -72,6 +74,10 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
       for (int r = 0; r < 2 * RP; ++r) daa[j][r] = 0.0f;
     }
 
+    // A word of this table that is neither frequent (side buffer) nor rare within the launch is
+    // written back by compare-and-swap; a rare one by a plain store (store_col16).
+    auto is_rare_word = [&](int w) { return w >= hot.n && is_rare(shadow, w); };
+
     // a B word that was a B word of an earlier row of this group is read only after that row's
     // delta has been added
     bool seen_before = false;
@@ -124,11 +130,13 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
             }
           }
         }
+        const uint32_t key = sr_key(seed, (uint32_t)i, (uint32_t)k);
         if (wb < hot.n)
           write_side_main<RP>(hot.sb, wb, dbb, lane, d);
+        else if (is_rare_word(wb))
+          store_col16<RP, ALIGNED>(B + (int64_t)wb * d, b, dbb, lane, d, key);
         else
-          add_col16<RP, ALIGNED>(B + (int64_t)wb * d, b, dbb, lane, d,
-                                 sr_key(seed, (uint32_t)i, (uint32_t)k));
+          add_col16<RP, ALIGNED>(B + (int64_t)wb * d, b, dbb, lane, d, key);
       }
       if (again) {
         wait_for_own_writes();
@@ -139,23 +147,33 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
     // the A columns, their exchanges in flight together
     {
       uint32_t ga_[MAXA][RP], fa_[MAXA][RP];
+      bool cas[MAXA];
 #pragma unroll
       for (int j = 0; j < MAXA; ++j) {
+        cas[j] = false;
         if (wa[j] >= 0) {
-          if (wa[j] < hot.n)
+          const uint32_t key = sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j);
+          // (a word that is an A word of the group twice keeps the exchange: two plain stores
+          // of "value read at the start of the group + delta" would keep only the second)
+          bool twice = false;
+#pragma unroll
+          for (int j2 = 0; j2 < MAXA; ++j2) twice = twice || (j2 != j && wa[j2] == wa[j]);
+          if (wa[j] < hot.n) {
             write_side_main<RP>(hot.sa, wa[j], daa[j], lane, d);
-          else if (ALIGNED)
-            cas_first<RP>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d,
-                          sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j), ga_[j], fa_[j]);
-          else
-            add_col16<RP, false>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d,
-                                 sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j));
+          } else if (!twice && is_rare_word(wa[j])) {
+            store_col16<RP, ALIGNED>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d, key);
+          } else if (ALIGNED) {
+            cas[j] = true;
+            cas_first<RP>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d, key, ga_[j], fa_[j]);
+          } else {
+            add_col16<RP, false>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d, key);
+          }
         }
       }
       if (ALIGNED) {
 #pragma unroll
         for (int j = 0; j < MAXA; ++j) {
-          if (wa[j] >= hot.n)   // implies wa[j] >= 0
+          if (cas[j])
             cas_rest<RP>(A + (int64_t)wa[j] * d, daa[j], lane, d,
                          sr_key(seed, (uint32_t)i, 0x10000U + (uint32_t)j), ga_[j], fa_[j]);
         }

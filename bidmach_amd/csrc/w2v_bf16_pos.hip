@@ -191,6 +191,7 @@ pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W
     const float ascale = scale_of(wi, vexp, smode);
     bool touched = false, a_written = false;
     const uint32_t akey = sr_key(seed, (uint32_t)i, 0U);
+    const bool a_rare = wi >= hot.n && is_rare(shadow, wi);
 
     const int base0 = min(jlo, -kLook);
     for (int base = base0; base <= jhi; base += kWave) {
@@ -233,9 +234,11 @@ pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W
           float gbs[CH];
           uint32_t guess[CH][RP], found[CH][RP];
           int wb[CH];
+          bool cas[CH];
 #pragma unroll
           for (int c = 0; c < CH; ++c) {
             wb[c] = -1;
+            cas[c] = false;
             if (c < nc) {
               wb[c] = read_lane(wl, src[c]);
               load_col16_fresh<RP, ALIGNED>(b[c], B + (int64_t)wb[c] * d, lane, d);
@@ -270,12 +273,18 @@ pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W
               }
               uint16_t* const bcol = B + (int64_t)wb[c] * d;
               const uint32_t key = sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c]));
-              if (wb[c] < hot.n)
+              cas[c] = false;
+              if (wb[c] < hot.n) {
                 write_side_main<RP>(hot.sb, wb[c], db, lane, d);
-              else if (ALIGNED)
+              } else if (is_rare(shadow, wb[c])) {
+                // rare within the launch: a plain store, nothing to wait for (store_col16)
+                store_col16<RP, ALIGNED>(bcol, b[c], db, lane, d, key);
+              } else if (ALIGNED) {
+                cas[c] = true;
                 cas_first<RP>(bcol, b[c], db, lane, d, key, guess[c], found[c]);
-              else
+              } else {
                 add_col16<RP, false>(bcol, b[c], db, lane, d, key);
+              }
             }
           }
           touched = true;
@@ -284,24 +293,29 @@ pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W
           const bool last = mask == 0ull && __ballot(ok && occ == round + 1) == 0ull &&
                             base + kWave > jhi;
           uint32_t aguess[RP], afound[RP];
+          bool acas = false;
           if (last) {
             a_written = true;
-            if (wi < hot.n)
+            if (wi < hot.n) {
               write_side_main<RP>(hot.sa, wi, daa, lane, d);
-            else if (ALIGNED)
+            } else if (a_rare) {
+              store_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
+            } else if (ALIGNED) {
+              acas = true;
               cas_first<RP>(acol, a, daa, lane, d, akey, aguess, afound);
-            else
+            } else {
               add_col16<RP, false>(acol, a, daa, lane, d, akey);
+            }
           }
           if (ALIGNED) {
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
-              if (wb[c] >= hot.n)   // implies c < nc
+              if (cas[c])
                 cas_rest_axpy<RP>(B + (int64_t)wb[c] * d, gbs[c], a, lane, d,
                                   sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c])), guess[c],
                                   found[c]);
             }
-            if (last && wi >= hot.n) cas_rest<RP>(acol, daa, lane, d, akey, aguess, afound);
+            if (acas) cas_rest<RP>(acol, daa, lane, d, akey, aguess, afound);
           }
         }
       }
@@ -310,6 +324,8 @@ pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W
       if (!a_written) {
         if (wi < hot.n)
           write_side_main<RP>(hot.sa, wi, daa, lane, d);
+        else if (a_rare)
+          store_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
         else
           add_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
       }
@@ -342,6 +358,10 @@ hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, con
   if (shadow.ordered != 0) {
     const int64_t chains = ordered_pos_chains(n, shift, kPosChainsBf16);
     const int64_t per_chain = ((int64_t)n + chains - 1) / chains;   // waves beyond: empty range
+    // words that are rare within the launch are written back with plain stores (store_col16)
+    lerr = prepare_rare_words(stream, W, n, nullptr, 0, 0x7fffffff, n, chains, &shadow,
+                              kRareCapOrderedBf16);
+    if (lerr != hipSuccess) return lerr;
     hipLaunchKernelGGL((pos_chain_bf16_kernel<RP, ALIGNED, PosChunk16<RP>::value>),
                        dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
                        dim3(kBlock), 0, stream, d, n, per_chain, W, LB, UB, A, B, lrate, vexp,

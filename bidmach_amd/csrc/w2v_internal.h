@@ -65,9 +65,10 @@ size_t read_copy_bytes();
 // Decides which words of a launch over `units` work units, `waves` of them in flight, are rare
 // enough for plain read-modify-write updates (Shadow::rare_max) and enqueues the count of the
 // words in the two id arrays (ids at or beyond idlimit are ignored).
+// cap: the largest number of occurrences that may still count as rare (0: the built-in 64).
 hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,
                               int64_t nb, int idlimit, int64_t units, int64_t waves,
-                              Shadow* shadow);
+                              Shadow* shadow, int cap = 0);
 // For kernels that only read: no shadow copies anywhere.
 inline Shadow no_shadow() {
   Shadow s{};
@@ -129,6 +130,9 @@ bool neg_rows_available(int nrows, int nwa);
 // asks for), within the bound on workgroups.
 constexpr int kNegRowWorkers = 576;        // fp32 row-by-row kernel, one row in flight per worker
 constexpr int kNegRowWorkersBf16 = 384;    // bfloat16 row-by-row kernel, which requests a row ahead
+// Ordered bfloat16 kernels: a word with at most this many occurrences in the launch is written back
+// with a plain store instead of a compare-and-swap (w2v_bf16.h, store_col16).
+constexpr int kRareCapOrderedBf16 = 16;
 constexpr int kPosTeams = 192;             // fp32 positive kernel, teams of kTeamWaves waves
 constexpr int kPosChainsBf16 = 128;        // bfloat16 positive kernel, single waves
 constexpr int kTeamWaves = 4;

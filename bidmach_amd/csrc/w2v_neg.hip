@@ -365,17 +365,18 @@ constexpr int kRareMaxCap = 64;
 constexpr int kRareMinSampledMax = 2;   // the scaled threshold is kept at or above this
 hipError_t prepare_rare_words(hipStream_t stream, const int* ids_a, int64_t na, const int* ids_b,
                               int64_t nb, int idlimit, int64_t units, int64_t waves,
-                              Shadow* shadow) {
+                              Shadow* shadow, int cap) {
   shadow->rare_max = 0;
   const int mode = g_rare_update_mode.load();
   if (mode == 0 || shadow->occurs == nullptr || waves <= 0) return hipSuccess;
   int64_t most = mode >= 2 ? mode : units / (kRareConcurrencyDen * waves);
-  if (most > kRareMaxCap) most = kRareMaxCap;
+  if (cap <= 0 || cap > kRareMaxCap) cap = kRareMaxCap;
+  if (most > cap) most = cap;
   if (most < 1) return hipSuccess;
   int every = 1;
   while (every < 8 && most / (2 * every) >= kRareMinSampledMax) every *= 2;
   // a sample needs something to sample from (forced thresholds on small calls)
-  while (every > 1 && (na < nb ? na : nb) / (16 * every) < 4096) every /= 2;
+  while (every > 1 && (nb > 0 && nb < na ? nb : na) / (16 * every) < 4096) every /= 2;
   const int sampled_max = (int)(most / every);
   hipLaunchKernelGGL(clear_occurs_kernel, dim3(256), dim3(kBlock), 0, stream,
                      reinterpret_cast<int4*>(shadow->occurs), kOccurSlots / 4);

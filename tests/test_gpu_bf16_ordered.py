@@ -132,3 +132,30 @@ def test_ordered_bf16_under_a_bound_on_workgroups(gpu, oracle, ordered, hot):
         b16.test_neg_update_bf16(gpu, oracle, hot, 0.0, 40, 70, 3, 40)   # the few-waves stand-in
     finally:
         ordered.w2v_set_max_workgroups(0)
+
+
+@pytest.fixture
+def rare_stores():
+    """Every word outside the side buffers counts as rare within the launch (forced threshold:
+    up to 64 occurrences), so the ordered kernels write it back with plain stores instead of
+    compare-and-swap exchanges (store_col16 in w2v_bf16.h)."""
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    assert lib.w2v_get_rare_update_mode() == -1
+    lib.w2v_set_rare_update_mode(64)
+    yield lib
+    lib.w2v_set_rare_update_mode(-1)
+
+
+@pytest.mark.parametrize("d,skip,ncentres", [(100, 5, 300), (300, 5, 300), (65, 3, 100)])
+def test_pos_update_bf16_ordered_with_plain_stores(gpu, oracle, ordered, rare_stores, hot, d, skip,
+                                                   ncentres):
+    """Without overlapping updates a plain store leaves the bits the exchange would."""
+    b16.test_pos_update_bf16(gpu, oracle, hot, 0.5, d, skip, ncentres)
+
+
+@pytest.mark.parametrize("d,nwa,nwb,G", [(100, 5, 5, 400), (300, 5, 5, 400), (65, 7, 8, 100),
+                                         (512, 15, 5, 100)])
+def test_neg_update_bf16_ordered_with_plain_stores(gpu, oracle, ordered, rare_stores, hot, d, nwa,
+                                                   nwb, G):
+    b16.test_neg_update_bf16(gpu, oracle, hot, 0.5, d, nwa, nwb, G)
