@@ -33,6 +33,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <atomic>
+#include <type_traits>
 
 #include "w2v_device.h"
 #include "w2v_internal.h"
@@ -844,35 +845,39 @@ constexpr int kHeavyPerLane = kHeavyBins / kHeavyThreads;   // bins a lane looks
 constexpr int kHeavyTop = kHotWords;
 static_assert(kHeavyWaves * kHeavyTop == kWave * kHeavyPerLane, "second stage: one wave, same shape");
 
-// The kHeavyTop largest of the kWave * kHeavyPerLane values a wave holds (v[k] of every lane),
-// largest first: out[r] is valid in every lane.  Wave-level only: no barrier.
+// Maximum over the 64 lanes, the same value in every lane: four DPP row rotations inside each
+// 16-lane row, then the four row maxima are read out (as wave_sum does for sums).
+__device__ __forceinline__ int wave_max(int x) {
+  auto rot = [](int v, auto ctrl) {
+    return __builtin_amdgcn_update_dpp(0, v, decltype(ctrl)::value, 0xf, 0xf, false);
+  };
+  x = max(x, rot(x, std::integral_constant<int, 0x128>{}));
+  x = max(x, rot(x, std::integral_constant<int, 0x124>{}));
+  x = max(x, rot(x, std::integral_constant<int, 0x122>{}));
+  x = max(x, rot(x, std::integral_constant<int, 0x121>{}));
+  return max(max(read_lane(x, 0), read_lane(x, 16)), max(read_lane(x, 32), read_lane(x, 48)));
+}
+
+// The kHeavyTop largest of the kWave * kHeavyPerLane counts a wave holds (v[k] of every lane,
+// each below 2^22), largest first: out[r] is valid in every lane.  A count travels with its place
+// (lane, k) in its low 8 bits, so every key is unique and the winner knows itself.  Wave-level
+// only: no barrier, no LDS.
 __device__ __forceinline__ void wave_top(int (&v)[kHeavyPerLane], int (&out)[kHeavyTop]) {
+  static_assert(kHeavyPerLane <= 4, "two bits for the place inside a lane");
   const int lane = threadIdx.x & 63;
+  int key[kHeavyPerLane];
+#pragma unroll
+  for (int k = 0; k < kHeavyPerLane; ++k) key[k] = v[k] < 0 ? -1 : (v[k] << 8) | (lane << 2) | k;
 #pragma unroll
   for (int r = 0; r < kHeavyTop; ++r) {
-    int best = -1, at = 0;
+    int best = -1;
 #pragma unroll
-    for (int k = 0; k < kHeavyPerLane; ++k) {
-      if (v[k] > best) {
-        best = v[k];
-        at = k;
-      }
-    }
-    int wbest = best, wlane = lane;
+    for (int k = 0; k < kHeavyPerLane; ++k) best = max(best, key[k]);
+    const int top = wave_max(best);
+    out[r] = top < 0 ? 0 : top >> 8;
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-      const int ov = __shfl_xor(wbest, m, kWave), ol = __shfl_xor(wlane, m, kWave);
-      if (ov > wbest || (ov == wbest && ol < wlane)) {
-        wbest = ov;
-        wlane = ol;
-      }
-    }
-    out[r] = wbest;
-    if (lane == wlane) {
-#pragma unroll
-      for (int k = 0; k < kHeavyPerLane; ++k)
-        if (k == at) v[k] = -1;
-    }
+    for (int k = 0; k < kHeavyPerLane; ++k)
+      if (key[k] == top) key[k] = -1;
   }
 }
 
