@@ -26,7 +26,7 @@ JNI_NAME = "libbidmachcuda-jni-linux-x86_64.so"
 JNI_PATH = os.path.join(LIB_DIR, JNI_NAME)
 
 SOURCES = ["w2v_pos.hip", "w2v_neg.hip", "w2v_neg_wide.hip", "w2v_neg_rows.hip", "w2v_any_shape.hip", "w2v_slice.hip", "w2v_wordmats.hip", "w2v_lz4.hip",
-           "w2v_bf16_pos.hip", "w2v_bf16_neg.hip", "w2v_bf16_neg_rows.hip", "w2v_bf16_neg_rows_unaligned.hip", "w2v_api.hip"]
+           "w2v_bf16_pos.hip", "w2v_bf16_pos_chain.hip", "w2v_bf16_neg.hip", "w2v_bf16_neg_rows.hip", "w2v_bf16_neg_rows_unaligned.hip", "w2v_api.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",

@@ -317,6 +317,29 @@ __device__ __forceinline__ void add_side_col(float (&x)[2 * RP], const float* si
   }
 }
 
+// The same in two steps, for callers that want several columns in flight before the first value
+// is used: side_col_request leaves the side column's values in s (zero beyond d), side_col_add adds
+// them.  (add_side_col uses each value as it names it, so a caller that gathers column after
+// column with it waits for every column before it asks for the next.)
+template <int RP>
+__device__ __forceinline__ void side_col_request(float (&s)[2 * RP], const float* side, int lane,
+                                                 int d) {
+#pragma unroll
+  for (int r = 0; r < 2 * RP; ++r) {
+    const int e = (r >> 1) * 128 + 2 * lane + (r & 1);
+    s[r] = 0.0f;
+    if (e < d)
+      s[r] = __hip_atomic_load(side + (r >> 1) * 128 + (r & 1) * 64 + lane, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int RP>
+__device__ __forceinline__ void side_col_add(float (&x)[2 * RP], const float (&s)[2 * RP]) {
+#pragma unroll
+  for (int r = 0; r < 2 * RP; ++r) x[r] += s[r];
+}
+
 template <int RP>
 __device__ __forceinline__ void atomic_add_side_col(float* side, const float (&delta)[2 * RP],
                                                     int lane, int d) {
@@ -353,18 +376,70 @@ __device__ __forceinline__ void read_side(float (&x)[2 * RP], const float* base,
   }
 }
 
-// The ordered kernels run a few hundred waves, too few for the extra copies to pay: they read and
-// write the main side column only (the end-of-call narrowing sums all copies either way).
-template <int RP>
-__device__ __forceinline__ void read_side_main(float (&x)[2 * RP], const float* base, int w,
-                                               int lane, int d) {
-  add_side_col<RP>(x, base + (int64_t)w * side_stride(d), lane, d);
+// The ordered kernels (a few hundred workers) read and write the main side column only, with one
+// exception: the row-by-row kernel of the negative pass uses the kTopCopies side columns of table
+// B's kTopWords most frequent words as a 2 x 2 grid of delta slots: slot g = 2 c + r is the main
+// column for g = 0 and extra column g - 1 otherwise; a writer adds its delta to both twins
+// r = 0, 1 of the copy c its worker number selects, a reader sums one twin r of both copies.
+// Every reader still sees every update made so far, and a column takes half of the adds and half
+// of the reads.  On a raw Zipf(1.1) stream one word is 13 % of the context words, and the
+// requests to its columns are served one after the other: from about 400 workers on the pass
+// does not get faster (55 ms per 1.2M groups at vocab 3M, with the slots 41 ms at 576 workers and
+// 37 ms at 768).  The positive kernel, whose workers are fewer, only pays for the second column
+// (teams of 160: 71 ms with the slots, 65 ms without) and stays with the main column.  The
+// end-of-call narrowing then sums twin 0 of both copies (fold_bf16_kernel).
+static_assert(kTopCopies == 4, "the ordered kernels lay the copies out as 2 x 2");
+
+__device__ __forceinline__ int64_t side_slot_column(int hot_n, int w, int g) {
+  return g == 0 ? (int64_t)w : (int64_t)hot_n + (g - 1) * kTopWords + w;
 }
 
+__device__ __forceinline__ bool has_side_slots(int hot_n, int w) {
+  return w < kTopWords && hot_n >= kTopWords;
+}
+
+// Requests what a reader of frequent word w needs (side_col_request: nothing is used yet): the
+// main side column into s, or twin r of both copies into s and s2.
+template <int RP>
+__device__ __forceinline__ void side_request_ordered(float (&s)[2 * RP], float (&s2)[2 * RP],
+                                                     const float* base, int hot_n, int w,
+                                                     int64_t worker, int lane, int d) {
+  const int64_t stride = side_stride(d);
+  if (has_side_slots(hot_n, w)) {
+    const int r = (int)(worker >> 1) & 1;
+    side_col_request<RP>(s, base + side_slot_column(hot_n, w, r) * stride, lane, d);
+    side_col_request<RP>(s2, base + side_slot_column(hot_n, w, 2 + r) * stride, lane, d);
+  } else {
+    side_col_request<RP>(s, base + (int64_t)w * stride, lane, d);
+  }
+}
+
+template <int RP>
+__device__ __forceinline__ void side_add_ordered(float (&x)[2 * RP], const float (&s)[2 * RP],
+                                                 const float (&s2)[2 * RP], int hot_n, int w) {
+  side_col_add<RP>(x, s);
+  if (has_side_slots(hot_n, w)) side_col_add<RP>(x, s2);
+}
+
+// Table A in the ordered kernels (the centre words and the negatives: no word takes a large
+// share of its updates) keeps to the main side column.
 template <int RP>
 __device__ __forceinline__ void write_side_main(float* base, int w, const float (&delta)[2 * RP],
                                                 int lane, int d) {
   atomic_add_side_col<RP>(base + (int64_t)w * side_stride(d), delta, lane, d);
+}
+
+template <int RP>
+__device__ __forceinline__ void write_side_ordered(float* base, int hot_n, int w, int64_t worker,
+                                                   const float (&delta)[2 * RP], int lane, int d) {
+  const int64_t stride = side_stride(d);
+  if (has_side_slots(hot_n, w)) {
+    const int c = (int)worker & 1;
+    atomic_add_side_col<RP>(base + side_slot_column(hot_n, w, 2 * c) * stride, delta, lane, d);
+    atomic_add_side_col<RP>(base + side_slot_column(hot_n, w, 2 * c + 1) * stride, delta, lane, d);
+  } else {
+    atomic_add_side_col<RP>(base + (int64_t)w * stride, delta, lane, d);
+  }
 }
 
 template <int RP>
@@ -394,6 +469,12 @@ hipError_t launch_pos_bf16(hipStream_t stream, int nrows, int ncols, int shift, 
 hipError_t launch_neg_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
                            const int* WA, const int* WB, uint16_t* A, uint16_t* B, float lrate,
                            float vexp, uint64_t seed, HotCols hot, Shadow shadow);
+// Ordered form of the positive pass (w2v_bf16_pos_chain.hip): counts the words that are rare
+// within the launch and enqueues the worker kernel; `aligned` as pair_aligned() found the tables.
+hipError_t launch_pos_chain_bf16(hipStream_t stream, int nrows, int ncols, int shift, const int* W,
+                                 const int* LB, const int* UB, uint16_t* A, uint16_t* B,
+                                 float lrate, float vexp, uint64_t seed, HotCols hot,
+                                 const Shadow& shadow, bool aligned);
 // Ordered form of the negative pass (w2v_bf16_neg_rows.hip); false if the shape has no instance.
 bool neg_rows_bf16_available(int nrows, int nwa);
 hipError_t launch_neg_rows_bf16(hipStream_t stream, int nrows, int ncols, int nwa, int nwb,
@@ -404,8 +485,10 @@ hipError_t launch_neg_rows_bf16_unaligned(hipStream_t stream, int nrows, int nco
                                           int nwb, const int* WA, const int* WB, uint16_t* A,
                                           uint16_t* B, float lrate, float vexp, uint64_t seed,
                                           HotCols hot, int64_t chains, const Shadow& shadow);
+// `slots_if_ordered`: the launch's ordered kernel (if the device-side decision is for it) used the
+// most frequent words' side columns as delta slots with twins (side_request_ordered).
 hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
-                            HotCols hot);
+                            HotCols hot, const Shadow& shadow, bool slots_if_ordered);
 // The forward twins add their sum into the device double Retval[0].
 hipError_t launch_eval_pos_bf16(hipStream_t stream, int nrows, int ncols, const int* W,
                                 const int* LB, const int* UB, const uint16_t* A,

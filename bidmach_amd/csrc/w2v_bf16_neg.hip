@@ -234,7 +234,7 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
     if (lerr != hipSuccess) return lerr;
   }
   if (hot.n == 0) return hipSuccess;
-  return launch_fold_bf16(stream, d, A, B, seed, hot);
+  return launch_fold_bf16(stream, d, A, B, seed, hot, shadow, rows);
 }
 
 template <bool ALIGNED, bool EVAL>

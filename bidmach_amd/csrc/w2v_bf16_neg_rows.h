@@ -39,13 +39,19 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
   const int64_t g_begin = chain * per_chain;
   const int64_t g_end = min(g_begin + per_chain, (int64_t)n);
 
-  auto load_a = [&](float (&x)[2 * RP], int word) {
+  // A column is requested here and used later: a frequent word's side column goes to registers
+  // of its own (`side`) and is added where the column is first used, so that several columns, or
+  // a row's column and the arithmetic of the row before it, are in flight together.
+  auto request_a = [&](float (&x)[2 * RP], float (&side)[2 * RP], int word) {
     load_col16_fresh<RP, ALIGNED>(x, A + (int64_t)word * d, lane, d);
-    if (word < hot.n) read_side_main<RP>(x, hot.sa, word, lane, d);
+    if (word < hot.n) side_col_request<RP>(side, hot.sa + (int64_t)word * side_stride(d), lane, d);
   };
-  auto load_b = [&](float (&x)[2 * RP], int word) {
+  // (table B holds the context words, the frequent ones of a raw stream: its most frequent words'
+  // side columns are read and written as delta slots, side_request_ordered)
+  auto request_b = [&](float (&x)[2 * RP], float (&side)[2 * RP], float (&side2)[2 * RP],
+                       int word) {
     load_col16_fresh<RP, ALIGNED>(x, B + (int64_t)word * d, lane, d);
-    if (word < hot.n) read_side_main<RP>(x, hot.sb, word, lane, d);
+    if (word < hot.n) side_request_ordered<RP>(side, side2, hot.sb, hot.n, word, chain, lane, d);
   };
 
   int wal = -1, wbl = -1;
@@ -63,20 +69,24 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
     const float sal = wa_l >= 0 ? scale_of(wa_l, vexp, smode) : 0.0f;
     const float sbl = wb_l >= 0 ? scale_of(wb_l, vexp, smode) : 0.0f;
 
+    // A word that is neither frequent (side buffer) nor rare within the launch is written back by
+    // compare-and-swap; a rare one by a plain store (store_col16).
+    // The counters of the group's words that may be rare within the launch are requested first
+    // and looked at after the columns have been requested (below): the other way round the
+    // columns would wait for the counters, or the counters for the columns.
+    const int seen_a = wa_l >= hot.n ? rare_seen(shadow, wa_l) : 0x7fffffff;
+    const int seen_b = wb_l >= hot.n ? rare_seen(shadow, wb_l) : 0x7fffffff;
+
     float a[MAXA][2 * RP], daa[MAXA][2 * RP];
     int wa[MAXA];
 #pragma unroll
     for (int j = 0; j < MAXA; ++j) {
       wa[j] = -1;
       if (j < nwa) wa[j] = read_lane(wa_l, j);
-      if (wa[j] >= 0) load_a(a[j], wa[j]);
-#pragma unroll
-      for (int r = 0; r < 2 * RP; ++r) daa[j][r] = 0.0f;
+      // (the side column of a frequent word waits in the registers of the column's delta, which
+      // are not needed before the first row)
+      if (wa[j] >= 0) request_a(a[j], daa[j], wa[j]);
     }
-
-    // A word of this table that is neither frequent (side buffer) nor rare within the launch is
-    // written back by compare-and-swap; a rare one by a plain store (store_col16).
-    auto is_rare_word = [&](int w) { return w >= hot.n && is_rare(shadow, w); };
 
     // a B word that was a B word of an earlier row of this group is read only after that row's
     // delta has been added
@@ -85,19 +95,29 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
       if (k < lane && read_lane(wb_l, k) == wb_l) seen_before = true;
     const unsigned long long repeats = __ballot(seen_before && wb_l >= 0);
 
-    float bn[2 * RP];
+    float bn[2 * RP], bnside[2 * RP], bnside2[2 * RP];
     int wbn = read_lane(wb_l, 0);
-    if (wbn >= 0) load_b(bn, wbn);
+    if (wbn >= 0) request_b(bn, bnside, bnside2, wbn);
+    const unsigned long long rare_a = __ballot(seen_a <= shadow.rare_max);
+    const unsigned long long rare_b = __ballot(seen_b <= shadow.rare_max);
+    // the A columns have been requested, and the first row's column: now their side columns
+#pragma unroll
+    for (int j = 0; j < MAXA; ++j) {
+      if (wa[j] >= 0 && wa[j] < hot.n) side_col_add<RP>(a[j], daa[j]);
+#pragma unroll
+      for (int r = 0; r < 2 * RP; ++r) daa[j][r] = 0.0f;
+    }
     for (int k = 0; k < nwb; ++k) {
       const int wb = wbn;
       float b[2 * RP];
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) b[r] = bn[r];
+      if (wb >= 0 && wb < hot.n) side_add_ordered<RP>(b, bnside, bnside2, hot.n, wb);
       bool again = false;
       if (k + 1 < nwb) {
         wbn = read_lane(wb_l, k + 1);
         again = wbn >= 0 && ((repeats >> (k + 1)) & 1ull) != 0;
-        if (wbn >= 0 && !again) load_b(bn, wbn);
+        if (wbn >= 0 && !again) request_b(bn, bnside, bnside2, wbn);
       }
       if (wb >= 0) {
         const float bs = read_lane(sbl, k);
@@ -132,15 +152,15 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
         }
         const uint32_t key = sr_key(seed, (uint32_t)i, (uint32_t)k);
         if (wb < hot.n)
-          write_side_main<RP>(hot.sb, wb, dbb, lane, d);
-        else if (is_rare_word(wb))
+          write_side_ordered<RP>(hot.sb, hot.n, wb, chain, dbb, lane, d);
+        else if ((rare_b >> k) & 1ull)
           store_col16<RP, ALIGNED>(B + (int64_t)wb * d, b, dbb, lane, d, key);
         else
           add_col16<RP, ALIGNED>(B + (int64_t)wb * d, b, dbb, lane, d, key);
       }
       if (again) {
         wait_for_own_writes();
-        load_b(bn, wbn);
+        request_b(bn, bnside, bnside2, wbn);
       }
     }
 
@@ -160,7 +180,7 @@ neg_rows_bf16_kernel(int d, int n, int64_t per_chain, int nwa, int nwb,
           for (int j2 = 0; j2 < MAXA; ++j2) twice = twice || (j2 != j && wa[j2] == wa[j]);
           if (wa[j] < hot.n) {
             write_side_main<RP>(hot.sa, wa[j], daa[j], lane, d);
-          } else if (!twice && is_rare_word(wa[j])) {
+          } else if (!twice && ((rare_a >> j) & 1ull)) {
             store_col16<RP, ALIGNED>(A + (int64_t)wa[j] * d, a[j], daa[j], lane, d, key);
           } else if (ALIGNED) {
             cas[j] = true;

@@ -127,214 +127,6 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
   }
 }
 
-// Ordered form of the update (launch_is_ordered, w2v_device.h): the token-by-token order of the
-// reference's CPU loop (BIDMach_CPUMACH.c:26-68) on a bounded number of workers, as
-// pos_chain_kernel (w2v_pos.hip) has it for fp32 tables.  A wave walks a contiguous range of
-// centre tokens one after the other; per token it reads the centre's A column and the window's B
-// columns with device-scope loads (table column plus the side buffer of a frequent word), writes
-// every B delta back at once - float atomics on the side buffer of a frequent word, else a
-// compare-and-swap with stochastic rounding, the exchanges of a chunk of columns in flight
-// together - and the A delta after the window, and waits for all of it before the next token's
-// reads.  A word that stands at several offsets of one window is worked on in rounds, occurrence
-// r after the writes of occurrence r - 1.  Every write uses the key of pos_bf16_kernel, so on a
-// minibatch without repeated words both kernels store the same bits.
-template <int RP>
-struct PosChunk16 {
-  // (larger chunks cost more registers than a wave has, and a spilled exchange result is waited
-  // for at once: 8 columns at dim 300 are slower than 4, 165 against 145 ms per 1M tokens)
-  static constexpr int value = RP <= 2 ? 8 : RP <= 6 ? 4 : 3;
-};
-
-template <int RP, bool ALIGNED, int CH>
-__global__ void __launch_bounds__(kBlock, 1)
-pos_chain_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
-                      const int* __restrict__ LB, const int* __restrict__ UB, uint16_t* A,
-                      uint16_t* B, float lrate, float vexp, int smode, uint64_t seed, HotCols hot,
-                      Shadow shadow_arg) {
-  const Shadow shadow = resolve_hot_mode(shadow_arg);
-  if (!launch_is_ordered(shadow_arg, shadow)) return;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t chain = (int64_t)blockIdx.x * kWavesPerBlock + wave;
-  const int64_t i_begin = chain * per_chain;
-  const int64_t i_end = min(i_begin + per_chain, (int64_t)n);
-
-  // the ids of the next token and of its window (offsets -32..31) are fetched while the current
-  // token is worked on
-  constexpr int kLook = 32;
-  int lb = 0, ub = 0, wnear = -1;
-  auto fetch = [&](int64_t t) {
-    lb = ub = 0;
-    wnear = -1;
-    if (t < i_end) {
-      lb = LB[t];
-      ub = UB[t];
-      const int64_t p = t + lane - kLook;
-      if (p >= 0 && p < n) wnear = W[p];
-    }
-  };
-  fetch(i_begin);
-  for (int64_t unit = i_begin; unit < i_end; ++unit) {
-    const int i = (int)unit;
-    const int wi = read_lane(wnear, kLook);
-    const int jlo = max(__builtin_amdgcn_readfirstlane(lb), -i);
-    const int jhi = min(__builtin_amdgcn_readfirstlane(ub), n - 1 - i);
-    const int wnear_now = wnear;
-    fetch(unit + 1);
-    if (wi < 0) continue;
-    uint16_t* const acol = A + (int64_t)wi * d;
-    float a[2 * RP], daa[2 * RP];
-    load_col16_fresh<RP, ALIGNED>(a, acol, lane, d);
-    if (wi < hot.n) read_side_main<RP>(a, hot.sa, wi, lane, d);
-#pragma unroll
-    for (int r = 0; r < 2 * RP; ++r) daa[r] = 0.0f;
-    const float ascale = scale_of(wi, vexp, smode);
-    bool touched = false, a_written = false;
-    const uint32_t akey = sr_key(seed, (uint32_t)i, 0U);
-    const bool a_rare = wi >= hot.n && is_rare(shadow, wi);
-
-    const int base0 = min(jlo, -kLook);
-    for (int base = base0; base <= jhi; base += kWave) {
-      // lane l looks at window offset base + l; the offsets -32..31 were fetched beforehand (a
-      // window wider than 64 offsets is worked on in slabs, each after the writes of the last)
-      if (base != base0) wait_for_own_writes();
-      const int j = base + lane;
-      int wl = -1;
-      if (j >= jlo && j <= jhi && j != 0) wl = base == -kLook ? wnear_now : W[i + j];
-      const bool ok = wl >= 0;
-      const float sl = ok ? scale_of(wl, vexp, smode) : 0.0f;
-      const unsigned long long valid = __ballot(ok);
-      int occ = 0;
-      {
-        unsigned long long m = valid;
-        while (m != 0ull) {
-          const int l = __builtin_ctzll(m);
-          m &= m - 1ull;
-          if (l < lane && read_lane(wl, l) == wl) ++occ;
-        }
-      }
-      for (int round = 0;; ++round) {
-        unsigned long long mask = __ballot(ok && occ == round);
-        if (mask == 0ull) break;
-        if (round > 0) wait_for_own_writes();
-        while (mask != 0ull) {
-          int src[CH];
-          int nc = 0;
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (mask != 0ull) {
-              src[c] = __builtin_ctzll(mask);
-              mask &= mask - 1ull;
-              nc = c + 1;
-            } else {
-              src[c] = -1;
-            }
-          }
-          float b[CH][2 * RP];
-          float gbs[CH];
-          uint32_t guess[CH][RP], found[CH][RP];
-          int wb[CH];
-          bool cas[CH];
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            wb[c] = -1;
-            cas[c] = false;
-            if (c < nc) {
-              wb[c] = read_lane(wl, src[c]);
-              load_col16_fresh<RP, ALIGNED>(b[c], B + (int64_t)wb[c] * d, lane, d);
-              if (wb[c] < hot.n) read_side_main<RP>(b[c], hot.sb, wb[c], lane, d);
-            }
-          }
-          // lane c forms the sigmoid of the dot with context c: one evaluation per chunk
-          float pre = 0.0f;
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (c < nc) {
-              float part = 0.0f;
-#pragma unroll
-              for (int r = 0; r < 2 * RP; ++r) part = fmaf(a[r], b[c][r], part);
-              const float sum = wave_sum(part);
-              pre = (lane == c) ? sum : pre;
-            }
-          }
-          const float gl = lrate * (1.0f - sat_sigmoid(pre));
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (c < nc) {
-              const float g = read_lane(gl, c);
-              const float ga = ascale * g;
-              const float gb = read_lane(sl, src[c]) * g;
-              gbs[c] = gb;
-              float db[2 * RP];
-#pragma unroll
-              for (int r = 0; r < 2 * RP; ++r) {
-                daa[r] = fmaf(ga, b[c][r], daa[r]);
-                db[r] = gb * a[r];
-              }
-              uint16_t* const bcol = B + (int64_t)wb[c] * d;
-              const uint32_t key = sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c]));
-              cas[c] = false;
-              if (wb[c] < hot.n) {
-                write_side_main<RP>(hot.sb, wb[c], db, lane, d);
-              } else if (is_rare(shadow, wb[c])) {
-                // rare within the launch: a plain store, nothing to wait for (store_col16)
-                store_col16<RP, ALIGNED>(bcol, b[c], db, lane, d, key);
-              } else if (ALIGNED) {
-                cas[c] = true;
-                cas_first<RP>(bcol, b[c], db, lane, d, key, guess[c], found[c]);
-              } else {
-                add_col16<RP, false>(bcol, b[c], db, lane, d, key);
-              }
-            }
-          }
-          touched = true;
-          // after the token's last chunk the centre's delta is complete: its exchange joins
-          // those of the chunk's columns in flight
-          const bool last = mask == 0ull && __ballot(ok && occ == round + 1) == 0ull &&
-                            base + kWave > jhi;
-          uint32_t aguess[RP], afound[RP];
-          bool acas = false;
-          if (last) {
-            a_written = true;
-            if (wi < hot.n) {
-              write_side_main<RP>(hot.sa, wi, daa, lane, d);
-            } else if (a_rare) {
-              store_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
-            } else if (ALIGNED) {
-              acas = true;
-              cas_first<RP>(acol, a, daa, lane, d, akey, aguess, afound);
-            } else {
-              add_col16<RP, false>(acol, a, daa, lane, d, akey);
-            }
-          }
-          if (ALIGNED) {
-#pragma unroll
-            for (int c = 0; c < CH; ++c) {
-              if (cas[c])
-                cas_rest_axpy<RP>(B + (int64_t)wb[c] * d, gbs[c], a, lane, d,
-                                  sr_key(seed, (uint32_t)i, (uint32_t)(base + src[c])), guess[c],
-                                  found[c]);
-            }
-            if (acas) cas_rest<RP>(acol, daa, lane, d, akey, aguess, afound);
-          }
-        }
-      }
-    }
-    if (touched) {
-      if (!a_written) {
-        if (wi < hot.n)
-          write_side_main<RP>(hot.sa, wi, daa, lane, d);
-        else if (a_rare)
-          store_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
-        else
-          add_col16<RP, ALIGNED>(acol, a, daa, lane, d, akey);
-      }
-      // the writes of this token are performed before the next token's columns are read
-      wait_for_own_writes();
-    }
-  }
-}
-
 template <int RP, bool ALIGNED, bool EVAL>
 hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, const int* LB,
                   const int* UB, uint16_t* A, uint16_t* B, float lrate, float vexp, uint64_t seed,
@@ -356,28 +148,25 @@ hipError_t launch(hipStream_t stream, int d, int n, int shift, const int* W, con
   hipError_t lerr = hipGetLastError();
   if (lerr != hipSuccess || EVAL) return lerr;
   if (shadow.ordered != 0) {
-    const int64_t chains = ordered_pos_chains(n, shift, kPosChainsBf16);
-    const int64_t per_chain = ((int64_t)n + chains - 1) / chains;   // waves beyond: empty range
-    // words that are rare within the launch are written back with plain stores (store_col16)
-    lerr = prepare_rare_words(stream, W, n, nullptr, 0, 0x7fffffff, n, chains, &shadow,
-                              kRareCapOrderedBf16);
-    if (lerr != hipSuccess) return lerr;
-    hipLaunchKernelGGL((pos_chain_bf16_kernel<RP, ALIGNED, PosChunk16<RP>::value>),
-                       dim3((unsigned)((chains + kWavesPerBlock - 1) / kWavesPerBlock)),
-                       dim3(kBlock), 0, stream, d, n, per_chain, W, LB, UB, A, B, lrate, vexp,
-                       scale_mode(vexp), seed, hot, shadow);
-    lerr = hipGetLastError();
+    lerr = launch_pos_chain_bf16(stream, d, n, shift, W, LB, UB, A, B, lrate, vexp, seed, hot,
+                                 shadow, ALIGNED);
     if (lerr != hipSuccess) return lerr;
   }
   if (hot.n == 0) return hipSuccess;
-  return launch_fold_bf16(stream, d, A, B, seed, hot);
+  return launch_fold_bf16(stream, d, A, B, seed, hot, shadow, false);
 }
 
 // One workgroup per frequent word and table: table column = narrow(widen(column) + side buffer),
 // side buffer = 0.  Elements whose side buffer is zero are left alone, so a word the call did not
-// update keeps its bits (and a word id beyond the vocabulary is never touched).
+// update keeps its bits (and a word id beyond the vocabulary is never touched).  The extra side
+// columns of the most frequent words are copies to be summed - unless the launch was run by an
+// ordered kernel, which uses them as delta slots with twins (side_request_ordered, w2v_bf16.h):
+// then the odd slots repeat the even ones and only the even ones count.
 __global__ void __launch_bounds__(kBlock)
-fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot) {
+fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot, Shadow shadow_arg,
+                 int slots_if_ordered) {
+  bool twins = false;
+  if (slots_if_ordered) twins = launch_is_ordered(shadow_arg, resolve_hot_mode(shadow_arg));
   const int w = blockIdx.x >> 1;
   const int table_b = blockIdx.x & 1;
   uint16_t* col = (table_b ? B : A) + (int64_t)w * d;
@@ -393,7 +182,7 @@ fold_bf16_kernel(int d, uint16_t* A, uint16_t* B, uint64_t seed, HotCols hot) {
     for (int c = 1; c < copies; ++c) {
       const float u = base[((int64_t)hot.n + (c - 1) * kTopWords + w) * stride + p];
       any = any || u != 0.0f;
-      v += u;
+      if (!(twins && (c & 1))) v += u;
     }
     if (any) {
       const float x = __builtin_bit_cast(float, (uint32_t)col[e] << 16) + v;
@@ -452,10 +241,10 @@ hipError_t launch_bf16_to_f32(hipStream_t stream, size_t n, const uint16_t* src,
 }
 
 hipError_t launch_fold_bf16(hipStream_t stream, int nrows, uint16_t* A, uint16_t* B, uint64_t seed,
-                            HotCols hot) {
+                            HotCols hot, const Shadow& shadow, bool slots_if_ordered) {
   if (hot.n <= 0) return hipSuccess;
   hipLaunchKernelGGL(fold_bf16_kernel, dim3(2u * (unsigned)hot.n), dim3(kBlock), 0, stream, nrows,
-                     A, B, seed, hot);
+                     A, B, seed, hot, shadow, slots_if_ordered ? 1 : 0);
   return hipGetLastError();
 }
 

@@ -266,6 +266,13 @@ __device__ __forceinline__ bool is_rare(const Shadow& sh, int w) {
   return sh.rare_max > 0 && w >= kHotWords && sh.occurs[w & (kOccurSlots - 1)] <= sh.rare_max;
 }
 
+// The same in two steps, for a worker that must not wait for the counter where it asks for it:
+// rare_seen requests the counter of word w (a value no threshold reaches if w cannot be rare),
+// and the word is rare if what arrives is at most sh.rare_max.
+__device__ __forceinline__ int rare_seen(const Shadow& sh, int w) {
+  return (sh.rare_max > 0 && w >= kHotWords) ? sh.occurs[w & (kOccurSlots - 1)] : 0x7fffffff;
+}
+
 // The mode a kernel runs in: the launcher's, unless the ids of this launch hold too few hot words
 // for shadow copies to pay (subsampled or re-numbered vocabularies), in which case every column is
 // read and updated in place.
@@ -329,6 +336,40 @@ __device__ __forceinline__ bool launch_is_cold(const Shadow& asked, const Shadow
 // is a device-scope atomic, performed at the memory side.)
 __device__ __forceinline__ void wait_for_own_writes() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
+
+// Teams of wavefronts in the ordered positive kernels (pos_chain_kernel, pos_team_bf16_kernel): a
+// wave's lanes look at the window offsets -kChainLook .. kChainLook - 1 of the centre token.
+constexpr int kChainLook = 32;
+
+// The wave of a team of `tw` (a power of two) that reads and writes the A column of word `w`.
+__device__ __forceinline__ int team_wave(int w, int tw) {
+  return (int)(((unsigned)w * 2654435761u) >> 16) & (tw - 1);
+}
+
+// A team deals the window's positions to its waves by their place in the token stream, so a
+// column is read and written by one wave while its position moves through consecutive windows,
+// and requests of one wave to one address are performed in order.  The order is NOT given where a
+// word that this token's window holds (and has just been updated by the wave of that position)
+// also stands at a position that only the next token's window reaches: the wave of that position
+// reads the column a fraction of a microsecond after the other wave's add was issued.  True if
+// that can happen, i.e. the team has to wait for its adds' acknowledgements before it goes on:
+// `wl` is the word this lane's position holds in this token's window (-1 if none), `wnear` the
+// word at the position whatever the window, `nlo`..`nhi` the next token's window (offsets of the
+// next token, clipped to the minibatch).  Conservative: any word the next window newly reaches
+// that this window holds anywhere counts, and so does a next window beyond the lanes' reach.
+__device__ __forceinline__ bool window_hands_over(int wl, int wnear, int lane, int nlo, int nhi) {
+  if (nlo < -kChainLook || nhi >= kChainLook - 1) return true;
+  const int jn = lane - kChainLook - 1;   // this lane's position as an offset of the next token
+  unsigned long long enter =
+      __ballot(wl < 0 && wnear >= 0 && jn >= nlo && jn <= nhi && jn != 0);
+  while (enter != 0ull) {
+    const int e = __builtin_ctzll(enter);
+    enter &= enter - 1ull;
+    const int we = __builtin_amdgcn_readlane(wnear, e);
+    if (__ballot(wl == we) != 0ull) return true;
+  }
+  return false;
 }
 
 // Whether this launch runs in its ordered form.  A launch that is full of frequent words (a raw,

@@ -135,6 +135,7 @@ constexpr int kNegRowWorkersBf16 = 384;    // bfloat16 row-by-row kernel, which 
 constexpr int kRareCapOrderedBf16 = 16;
 constexpr int kPosTeams = 192;             // fp32 positive kernel, teams of kTeamWaves waves
 constexpr int kPosChainsBf16 = 128;        // bfloat16 positive kernel, single waves
+constexpr int kPosTeamsBf16 = 160;         // bfloat16 positive kernel, teams of kTeamWaves waves
 constexpr int kTeamWaves = 4;
 int64_t ordered_neg_chains(int waves_per_wg, int builtin);
 int64_t ordered_pos_chains(int ncols, int shift, int builtin);

@@ -234,19 +234,14 @@ pos_eval_kernel(int d, int ncols, int64_t units_per_wg, const int* __restrict__ 
 // whose updates the others do not see), so what is left to make the pass faster is the time a
 // worker spends on a token: a random 1.2 KB column takes about 2 us to arrive, and a wave issues
 // the float atomics of one column in about 0.35 us.  A worker is therefore a TEAM of TW
-// wavefronts (a workgroup): the window's words are dealt to the waves by a hash of the word id,
-// each wave gathers, dots and updates the B columns of its words, the centre's column is read
-// by the wave that owns the centre's word and handed round in LDS, and the waves' shares of the
-// centre's delta meet in LDS and are added by that same wave.  A column is only ever read and
-// written by the one wave of a team that its word hashes to, so a team's accesses to one column
-// stay in program order (requests of one wave to one address are performed in order; requests of
-// different waves need not be), and one team reproduces the sequential result exactly.
-constexpr int kChainLook = 32;
-
-// The wave of a team of `tw` (a power of two) that owns word `w`.
-__device__ __forceinline__ int team_wave(int w, int tw) {
-  return (int)(((unsigned)w * 2654435761u) >> 16) & (tw - 1);
-}
+// wavefronts (a workgroup): the window's positions are dealt to the waves by their place in the
+// token stream, each wave gathers, dots and updates the B columns of its positions, the centre's
+// column is read by the wave that the centre's word hashes to (team_wave) and handed round in
+// LDS, and the waves' shares of the centre's delta meet in LDS and are added by that same wave.
+// A position stays with one wave while it moves through consecutive windows, and requests of one
+// wave to one address are performed in order (requests of different waves need not be); where a
+// column goes from one wave to another (a word at several positions, window_hands_over) the
+// team waits for its adds' acknowledgements first, so one team reproduces the sequential result.
 
 // One centre token worked on by one wave alone: window offsets of any reach, in slabs of 64.
 // `wnear` holds the word ids at offsets -32..31 of token i (lane l: offset l - 32).
@@ -523,9 +518,17 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
 #pragma unroll
     for (int r = 0; r < R; ++r) s_da[wave][r * kWave + lane] = daa[r];
     // The next reader of a word that stands at several positions may be another wave (when its
-    // first position leaves the window): this wave's adds have been performed before the team
-    // goes on
-    if (repeats) __builtin_amdgcn_s_waitcnt(0);
+    // first position leaves the window), and so may the reader of a word that the next token's
+    // window meets again at a new position (window_hands_over), or of any word after a token that
+    // is skipped: then this wave's adds have been performed before the team goes on
+    bool settle = repeats;
+    if (!settle && unit + 1 < i_end) {
+      const int wn = read_lane(wnear_now, kChainLook + 1);
+      const int nlo = max(__builtin_amdgcn_readfirstlane(lb), -(i + 1));
+      const int nhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 2 - i);
+      settle = tables.a(wn, d).flags == 0 || window_hands_over(wl, wnear_now, lane, nlo, nhi);
+    }
+    if (settle) __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (wave == oa && tables.written(pa.flags)) {
       zero_col<R>(daa);
@@ -833,12 +836,14 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
 // the n ids of the launch, are left where the update kernels look for "the ids among the 16 most
 // frequent words" and "the most frequent word" (Shadow::hot_seen: four arrays of kHotCountSlots
 // partial counts; the values go to slot 0, the other slots are zeroed); the same for `ids2` (the
-// words read from table A; null: not counted).  Two frequent words that share a bin only make the
-// largest bin larger, and the words that are not frequent add about four ids to every bin, 0.4 %
-// of the sample over the kHeavyTop bins: both err towards "frequent".  One workgroup.
+// words read from table A; null: not counted).  The words that are not frequent add about eight
+// ids to every bin (0.4 % of the sample over the kHeavyTop bins, enough to tip a stream that is
+// just below the line): the mean of the other bins is taken off each of the largest.  Two
+// frequent words that share a bin only make the largest bin larger, which errs towards
+// "frequent".  The sample's own noise is 0.13 % of the ids at a share of 6 %.  One workgroup.
 constexpr int kHeavyThreads = 1024;
 constexpr int kHeavyWaves = kHeavyThreads / kWave;
-constexpr int kHeavySamples = 16384;
+constexpr int kHeavySamples = 32768;
 constexpr int kHeavyPerThread = kHeavySamples / kHeavyThreads;
 constexpr int kHeavyBins = 4096;
 constexpr int kHeavyPerLane = kHeavyBins / kHeavyThreads;   // bins a lane looks after
@@ -887,11 +892,13 @@ count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict
   __shared__ int s_bins[kHeavyBins];
   __shared__ int s_cand[kHeavyWaves * kHeavyTop];
   __shared__ long long s_result[2];
+  __shared__ int s_binned;
   const int tid = threadIdx.x;
   for (int which = 0; which < 2; ++which) {
     const int* const p = which ? ids2 : ids;
     const int64_t len = which ? n2 : n;
     if (tid < 2) s_result[tid] = 0;
+    if (tid == 0) s_binned = 0;
     if (p != nullptr && len > 0) {
       for (int k = tid; k < kHeavyBins; k += kHeavyThreads) s_bins[k] = 0;
       __syncthreads();
@@ -903,9 +910,15 @@ count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict
         const int64_t at = (int64_t)k * kHeavyThreads + tid;
         w[k] = at < nsamp ? p[at * stride] : -1;
       }
+      int binned = 0;
 #pragma unroll
-      for (int k = 0; k < kHeavyPerThread; ++k)
-        if (w[k] >= 0) atomicAdd(&s_bins[((unsigned)w[k] * 2654435761u) >> 20], 1);
+      for (int k = 0; k < kHeavyPerThread; ++k) {
+        if (w[k] >= 0) {
+          atomicAdd(&s_bins[((unsigned)w[k] * 2654435761u) >> 20], 1);
+          ++binned;
+        }
+      }
+      if (binned > 0) atomicAdd(&s_binned, binned);
       __syncthreads();
       // every wave picks the largest of its 256 bins, then the first wave the largest of those
       int v[kHeavyPerLane], top[kHeavyTop];
@@ -925,9 +938,13 @@ count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict
           long long sum = 0;
 #pragma unroll
           for (int r = 0; r < kHeavyTop; ++r) sum += top[r] > 0 ? top[r] : 0;
+          // what the words that are not frequent leave in a bin: the mean of the other bins
+          const double rest = (double)(s_binned - sum) / (double)(kHeavyBins - kHeavyTop);
+          const double top_sum = fmax((double)sum - kHeavyTop * rest, 0.0);
+          const double top_one = fmax((double)(top[0] > 0 ? top[0] : 0) - rest, 0.0);
           // sampled counts scaled up to the whole array (dropped words, id < 0, stay in the total)
-          s_result[0] = sum * len / nsamp;
-          s_result[1] = (long long)(top[0] > 0 ? top[0] : 0) * len / nsamp;
+          s_result[0] = (long long)(top_sum * (double)len / (double)nsamp);
+          s_result[1] = (long long)(top_one * (double)len / (double)nsamp);
         }
       }
     }

@@ -96,6 +96,50 @@ def test_one_worker_reproduces_the_sequential_positive_pass(gpu, oracle, d, skip
     assert max(np.abs(At - Ao).max(), np.abs(Bt - Bo).max()) > 50 * err + 1e-3
 
 
+def comes_back_stream(rng, n, skip, fixed):
+    """Distinct words, except that word 3 stands at every (2 skip + 1)-th position: it leaves
+    a token's window at one end just as the next token's window reaches its next occurrence at
+    the other end, which inside a team of wavefronts is another wave's position."""
+    W = (16 + rng.permutation(n)).astype(np.int32)
+    W[7::2 * skip + 1] = 3
+    if fixed:
+        LB = np.full(n, -skip, np.int32)
+        UB = np.full(n, skip, np.int32)
+    else:
+        LB, UB = corpus.window_bounds(n, skip, rng)
+    return W, LB, UB
+
+
+@pytest.mark.parametrize("fixed", [True, False])
+@pytest.mark.parametrize("d,skip", [(100, 5), (300, 5), (64, 3)])
+def test_one_team_hands_a_column_from_wave_to_wave_in_order(gpu, oracle, d, skip, fixed):
+    """One worker (a team of four wavefronts) on a stream whose only repeated word comes back one
+    position beyond the window each time: the wave that reads its column for the next token is
+    not the wave that has just added to it, and must still see that add (the sequential oracle's
+    result, up to the rounding of the dot products; a missed add is 1e-3 and more)."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(d + skip)
+    n = 600
+    V = n + 16
+    A = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    B = (rng.standard_normal((V, d)) * 0.3).astype(np.float32)
+    W, LB, UB = comes_back_stream(rng, n, skip, fixed)
+    Ao, Bo = A.copy(), B.copy()
+    oracle.word2vecPos(d, n, skip, W, LB, UB, Ao, Bo, 0.05, 0.0, 1)
+    lib.w2v_set_ordered_mode(1)
+    lib.w2v_set_ordered_workers(1, 1)
+    try:
+        Ag, Bg = parity.gpu_pos(gpu, d, skip, W, LB, UB, A, B, 0.05, 0.0)
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+        lib.w2v_set_ordered_workers(0, 0)
+    err = max(np.abs(Ag - Ao).max(), np.abs(Bg - Bo).max())
+    assert np.abs(Bo[3] - B[3]).max() > 0.05     # the word's column did move, many times
+    assert err <= 2e-5, err
+
+
 @pytest.mark.parametrize("d,nwa,nwb", [(100, 5, 5), (300, 5, 5), (200, 12, 3), (300, 5, 10),
                                        (100, 3, 14)])
 def test_one_worker_reproduces_the_sequential_negative_pass(gpu, oracle, d, nwa, nwb):
