@@ -190,7 +190,7 @@ def parse_args():
                          "default: the library's own numbers)")
     ap.add_argument("--ordered-copies", default="",
                     help="w2v_set_ordered_copies as COPIES,TWINS (delta slots of the 16 most "
-                         "frequent columns in the ordered kernels; default: the library's 4,4)")
+                         "frequent columns in the ordered kernels; default: the library's 2,2)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pcie", action="store_true",
                     help="skip the extra leg that uploads the index arrays from the host each step")

@@ -266,6 +266,15 @@ __device__ __forceinline__ bool is_rare(const Shadow& sh, int w) {
   return sh.rare_max > 0 && w >= kHotWords && sh.occurs[w & (kOccurSlots - 1)] <= sh.rare_max;
 }
 
+// The throughput kernels hold a rare A column between its read and its write for the time of a
+// chunk of dot products and cannot shorten that by reading it again, as they do for the B columns
+// (neg_train_kernel): the A words are held to a limit one count lower, which takes their lost
+// share of all contributions below that of the B words.
+__device__ __forceinline__ bool is_rare_a(const Shadow& sh, int w) {
+  const int limit = sh.rare_max > 1 ? sh.rare_max - 1 : sh.rare_max;
+  return sh.rare_max > 0 && w >= kHotWords && sh.occurs[w & (kOccurSlots - 1)] <= limit;
+}
+
 // The same in two steps, for a worker that must not wait for the counter where it asks for it:
 // rare_seen requests the counter of word w (a value no threshold reaches if w cannot be rare),
 // and the word is rare if what arrives is at most sh.rare_max.
@@ -347,27 +356,38 @@ __device__ __forceinline__ int team_wave(int w, int tw) {
   return (int)(((unsigned)w * 2654435761u) >> 16) & (tw - 1);
 }
 
-// A team deals the window's positions to its waves by their place in the token stream, so a
+// A team deals the window's positions to its waves by their place in the token stream (a word
+// that stands at several positions belongs, with all of them, to the wave of the first), so a
 // column is read and written by one wave while its position moves through consecutive windows,
-// and requests of one wave to one address are performed in order.  The order is NOT given where a
-// word that this token's window holds (and has just been updated by the wave of that position)
-// also stands at a position that only the next token's window reaches: the wave of that position
-// reads the column a fraction of a microsecond after the other wave's add was issued.  True if
-// that can happen, i.e. the team has to wait for its adds' acknowledgements before it goes on:
-// `wl` is the word this lane's position holds in this token's window (-1 if none), `wnear` the
-// word at the position whatever the window, `nlo`..`nhi` the next token's window (offsets of the
-// next token, clipped to the minibatch).  Conservative: any word the next window newly reaches
-// that this window holds anywhere counts, and so does a next window beyond the lanes' reach.
-__device__ __forceinline__ bool window_hands_over(int wl, int wnear, int lane, int nlo, int nhi) {
+// and requests of one wave to one address are performed in order.  The order is NOT given where
+// a word that this token's window holds, and that has just been updated by the wave of its
+// position, belongs to another wave in the next token's window: that wave reads the column a
+// fraction of a microsecond after the other wave's add was issued.  True if that can happen, i.e.
+// the team has to wait for its adds' acknowledgements before it goes on.  `wl` is the word this
+// lane's position holds in this token's window (-1 if none), `wnear` the word at the position
+// whatever the window, `nlo`..`nhi` the next token's window (offsets of the next token, clipped
+// to the minibatch), `tw` the team's waves.  Only words with one occurrence in this window are
+// looked at (after a window with a repeated word the team waits anyway): such a word changes
+// hands if a position that the next window newly reaches holds it and becomes its first
+// position there, on another wave - because the old position has left the window, or the new
+// one lies before it.  A next window beyond the lanes' reach counts as a change of hands.
+__device__ __forceinline__ bool window_hands_over(int wl, int wnear, int lane, int nlo, int nhi,
+                                                  int tw) {
   if (nlo < -kChainLook || nhi >= kChainLook - 1) return true;
   const int jn = lane - kChainLook - 1;   // this lane's position as an offset of the next token
-  unsigned long long enter =
-      __ballot(wl < 0 && wnear >= 0 && jn >= nlo && jn <= nhi && jn != 0);
+  const bool in_next = jn >= nlo && jn <= nhi && jn != 0;
+  const unsigned long long stays = __ballot(wl >= 0 && in_next);
+  unsigned long long enter = __ballot(wl < 0 && wnear >= 0 && in_next);
   while (enter != 0ull) {
     const int e = __builtin_ctzll(enter);
     enter &= enter - 1ull;
     const int we = __builtin_amdgcn_readlane(wnear, e);
-    if (__ballot(wl == we) != 0ull) return true;
+    const unsigned long long held = __ballot(wl == we);
+    if (held != 0ull) {
+      const int p = __builtin_ctzll(held);           // its (first) position in this window
+      const bool keeps = ((stays >> p) & 1ull) != 0 && p < e;   // still first in the next window
+      if (!keeps && ((p ^ e) & (tw - 1)) != 0) return true;
+    }
   }
   return false;
 }

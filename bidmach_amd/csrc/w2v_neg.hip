@@ -210,7 +210,7 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       // (an A word updated on several trips is not rare: its plain updates would be in flight
       // together)
       const uint64_t rare_a =
-          __ballot(wal >= 0 && lone_a && nwb <= MAXB && is_rare(shadow, wal));
+          __ballot(wal >= 0 && lone_a && nwb <= MAXB && is_rare_a(shadow, wal));
       const unsigned tka = hot_ticket(shadow, 1, slot, (wal >= 0 && wal < kHotWords) ? wal : -1);
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -268,6 +268,15 @@ neg_train_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t grou
       }
     }
 
+    // A rare B column was read when the group began, a whole group's work ago: it is read
+    // again now (into the registers of the old value, which no dot needs any more), so that what
+    // another wave wrote to it in the meantime is kept and only a write that falls into the last
+    // few microseconds can be lost.
+#pragma unroll
+    for (int k = 0; k < MAXB; ++k) {
+      if (wb[k] >= 0 && ((rare_b >> (kb + k)) & 1))
+        load_col_fresh<R>(b[k], B + (int64_t)wb[k] * d, lane, d);
+    }
 #pragma unroll
     for (int k = 0; k < MAXB; ++k) {
       if (wb[k] >= 0) {

@@ -364,17 +364,28 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
   const int64_t i_begin = chain * per_chain;
   const int64_t i_end = min(i_begin + per_chain, (int64_t)ncols);
 
-  int lb = 0, ub = 0, wnear = -1;
+  // Word ids of token t and of its window; the window bounds are requested one token further
+  // ahead (those of token t were asked for with token t - 1), so that a token also knows its
+  // successor's window without waiting for anything it has just asked for.
+  int lb = 0, ub = 0, lbn = 0, ubn = 0, wnear = -1;
   auto fetch = [&](int64_t t) {
-    lb = ub = 0;
+    lb = lbn;
+    ub = ubn;
+    lbn = ubn = 0;
     wnear = -1;
     if (t < i_end) {
-      lb = LB[t];
-      ub = UB[t];
       const int64_t p = t + lane - kChainLook;
       if (p >= 0 && p < ncols) wnear = W[p];
     }
+    if (t + 1 < i_end) {
+      lbn = LB[t + 1];
+      ubn = UB[t + 1];
+    }
   };
+  if (i_begin < i_end) {
+    lbn = LB[i_begin];
+    ubn = UB[i_begin];
+  }
   fetch(i_begin);
   for (int64_t unit = i_begin; unit < i_end; ++unit) {
     const int i = (int)unit;
@@ -382,6 +393,8 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     const int jlo = max(__builtin_amdgcn_readfirstlane(lb), -i);
     const int jhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 1 - i);
     const int wnear_now = wnear;
+    const int nlb = __builtin_amdgcn_readfirstlane(lbn);   // the next token's bounds
+    const int nub = __builtin_amdgcn_readfirstlane(ubn);
     fetch(unit + 1);
     const ColRef pa = tables.a(wi, d);
     if (pa.flags == 0) continue;
@@ -419,15 +432,18 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // to the wave of its first position, and occurrence number r of it is worked on in round r
     // (see chain_token_solo).
     int occ = 0, first = lane;
+    bool met = false;   // the word at this lane's position stands in the window (elsewhere)
     {
       unsigned long long m = valid;
       while (m != 0ull) {
         const int l = __builtin_ctzll(m);
         m &= m - 1ull;
-        if (l < lane && read_lane(wl, l) == wl) {
+        const int w_l = read_lane(wl, l);
+        if (l < lane && w_l == wl) {
           if (occ == 0) first = l;
           ++occ;
         }
+        met = met || (l != lane && w_l == wnear_now);
       }
     }
     const bool mine = ok && ((i + first) & (TW - 1)) == wave;
@@ -491,6 +507,24 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // the first columns of this wave are requested before the centre's column is handed round
     unsigned long long mask = __ballot(mine && occ == 0);
     gather(mask);
+    // (worked out here, under the wait for the columns just requested)
+    bool settle = repeats;
+#ifndef W2V_PROBE_NO_HANDOVER
+    if (!settle && unit + 1 < i_end) {
+      const int wn = read_lane(wnear_now, kChainLook + 1);
+      const int nlo = max(nlb, -(i + 1));
+      const int nhi = min(nub, ncols - 2 - i);
+      if (tables.a(wn, d).flags == 0 || nlo < -kChainLook || nhi >= kChainLook - 1) {
+        settle = true;
+      } else {
+        // (most tokens end here: no position that the next window newly reaches holds a word of
+        // this window)
+        const int jn = lane - kChainLook - 1;
+        if (__ballot(met && wl < 0 && jn >= nlo && jn <= nhi && jn != 0) != 0ull)
+          settle = window_hands_over(wl, wnear_now, lane, nlo, nhi, TW);
+      }
+    }
+#endif
     if (wave == oa) {
 #pragma unroll
       for (int r = 0; r < R; ++r) s_a[r * kWave + lane] = a[r];
@@ -521,14 +555,12 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // first position leaves the window), and so may the reader of a word that the next token's
     // window meets again at a new position (window_hands_over), or of any word after a token that
     // is skipped: then this wave's adds have been performed before the team goes on
-    bool settle = repeats;
-    if (!settle && unit + 1 < i_end) {
-      const int wn = read_lane(wnear_now, kChainLook + 1);
-      const int nlo = max(__builtin_amdgcn_readfirstlane(lb), -(i + 1));
-      const int nhi = min(__builtin_amdgcn_readfirstlane(ub), ncols - 2 - i);
-      settle = tables.a(wn, d).flags == 0 || window_hands_over(wl, wnear_now, lane, nlo, nhi);
-    }
+#ifdef W2V_PROBE_NO_WAIT
+    if (settle && !repeats) asm volatile("s_nop 0");
+    if (repeats) __builtin_amdgcn_s_waitcnt(0);
+#else
     if (settle) __builtin_amdgcn_s_waitcnt(0);
+#endif
     __syncthreads();
     if (wave == oa && tables.written(pa.flags)) {
       zero_col<R>(daa);

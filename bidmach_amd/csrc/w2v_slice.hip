@@ -211,7 +211,7 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg_all,
         for (int j = 0; j < jend; ++j)
           if (j != lane && read_lane(wal, j) == wal) lone = false;
         rare_a = __ballot(lone && nwb <= MAXB && pal.hot < 0 && tables.written(pal.flags) &&
-                          is_rare(shadow, wal));
+                          is_rare_a(shadow, wal));
       }
 
       for (int j0 = 0; j0 < jend; j0 += CHA) {
@@ -279,6 +279,12 @@ slice_neg_kernel(int d, int ngroups, int nwa, int nwb, int64_t units_per_wg_all,
     }
 
     if (TRAIN) {
+      // a rare B column is read again just before its plain store (see neg_train_kernel)
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k) {
+        if (kb + k < nwb && ((rare_b >> (kb + k)) & 1))
+          load_col_fresh<R>(b[k], rb[k].col, lane, d);
+      }
 #pragma unroll
       for (int k = 0; k < MAXB; ++k) {
         if (kb + k < nwb && ((rare_b >> (kb + k)) & 1))

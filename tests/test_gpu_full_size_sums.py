@@ -147,12 +147,13 @@ def test_subsampled_stream_default_settings(gpu, tables):
     """After the reference caller's frequent-word subsampling the launch holds no frequent words
     and the default is the throughput kernels, rare-word plain updates included.  Here most
     updates belong to words that are rare within the call, so the plain updates carry most of
-    the pass, and what they lose is a larger share than on the raw stream.  Measured (dim 32 and
-    dim 300 alike): 0.8-1.1 % of the A rows and 1.9-2.2 % of the B rows miss an update, 0.2-0.3 %
-    and 0.6-0.7 % of the contributions (w2v_set_rare_update_mode(0) keeps every one, at 6.1 ms
-    instead of 4.4 ms for the pass; a limit of 6 occurrences: 0.1 %, 4.9 ms).  The held-out loss
-    of this regime is within 0.01 % of the oracle's with the default
-    (tests/test_gpu_training.py)."""
+    the pass, and what they lose is a larger share than on the raw stream.  A rare B column is
+    read again just before it is written (the group's work lies between its first read and its
+    write), and the A words are held to a lower limit: measured (dim 32 and dim 300 alike)
+    1.1 % of the A rows miss an update, 0.22 % of the A contributions and 0.11 % of the B
+    contributions (0.3 % and 0.7 % before those two changes; w2v_set_rare_update_mode(0) keeps
+    every one, at 6.1 ms instead of 4.7 ms for the pass).  The held-out loss of this regime is
+    within 0.01 % of the oracle's with the default (tests/test_gpu_training.py)."""
     W, LB, UB, WA, WB, G = stream(1.0e-4)
     assert G > 400_000
     for what, (got, want) in run_both_ways(gpu, tables, W, LB, UB, WA, WB, G).items():
@@ -160,7 +161,7 @@ def test_subsampled_stream_default_settings(gpu, tables):
         if what.startswith("pos"):
             assert rel.max() <= 1e-3
         assert (rel > 1e-3).mean() <= 0.05
-        assert -1e-4 <= missing <= 1.5e-2
+        assert -1e-4 <= missing <= 3e-3
 
 
 def test_sliced_negative_pass_at_full_size(gpu, tables):
