@@ -276,6 +276,7 @@ pos_team_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
   // the centre's column as its owner read it, and each wave's share of the centre's delta
   __shared__ float s_a[2 * RP * kWave];
   __shared__ float s_da[TW][2 * RP * kWave];
+  __shared__ int s_hands;   // the team waits for its writes before the next token (see below)
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
   const int lane = threadIdx.x & (kWave - 1);
@@ -347,18 +348,15 @@ pos_team_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
     // that stands at several positions of the window belongs, with all of them, to the wave of
     // its first position, and occurrence number r of it is worked on in round r.
     int occ = 0, first = lane;
-    bool met = false;   // the word at this lane's position stands in the window (elsewhere)
     {
       unsigned long long m = valid;
       while (m != 0ull) {
         const int l = __builtin_ctzll(m);
         m &= m - 1ull;
-        const int w_l = read_lane(wl, l);
-        if (l < lane && w_l == wl) {
+        if (l < lane && read_lane(wl, l) == wl) {
           if (occ == 0) first = l;
           ++occ;
         }
-        met = met || (l != lane && w_l == wnear_now);
       }
     }
     const bool mine = ok && ((i + first) & (TW - 1)) == wave;
@@ -473,24 +471,20 @@ pos_team_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
     // the first columns of this wave are requested before the centre's column is handed round
     unsigned long long mask = __ballot(mine && occ == 0);
     gather(mask);
-    // (worked out here, under the wait for the columns just requested)
-    bool settle = repeats;
-#ifndef W2V_PROBE_NO_HANDOVER
-    if (!settle && unit + 1 < i_end) {
-      const int wn = read_lane(wnear_now, kChainLook + 1);
-      const int nlo = max(nlb, -(i + 1));
-      const int nhi = min(nub, n - 2 - i);
-      if (wn < 0 || nlo < -kChainLook || nhi >= kChainLook - 1) {
-        settle = true;
-      } else {
-        // (most tokens end here: no position that the next window newly reaches holds a word of
-        // this window)
-        const int jn = lane - kChainLook - 1;
-        if (__ballot(met && wl < 0 && jn >= nlo && jn <= nhi && jn != 0) != 0ull)
-          settle = window_hands_over(wl, wnear_now, lane, nlo, nhi, TW);
+    // Whether a column passes to another wave with the next token (window_hands_over): worked
+    // out by one wave that is not the centre's, which would otherwise only wait at the barrier
+    // for the centre's column, from what the token knew when it began, and handed round in LDS.
+    if (wave == ((oa + 1) & (TW - 1))) {
+      bool hands = false;
+      if (!repeats && unit + 1 < i_end) {
+        const int wn = read_lane(wnear_now, kChainLook + 1);
+        const int nlo = max(nlb, -(i + 1));
+        const int nhi = min(nub, n - 2 - i);
+        hands = wn < 0 || nlo < -kChainLook || nhi >= kChainLook - 1 ||
+                window_hands_over(wl, wnear_now, lane, nlo, nhi, TW);
       }
+      if (lane == 0) s_hands = hands ? 1 : 0;
     }
-#endif
     if (wave == oa) {
       if (wi < hot.n) side_col_add<RP>(a, aside);
 #pragma unroll
@@ -525,7 +519,7 @@ pos_team_bf16_kernel(int d, int n, int64_t per_chain, const int* __restrict__ W,
     // first one leaves the window; a word that the next token's window meets again at a new
     // position, window_hands_over; any word after a token that is skipped), this wave's writes
     // have been performed before the team goes on
-    if (settle) __builtin_amdgcn_s_waitcnt(0);
+    if (repeats || s_hands != 0) __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (wave == oa) {
 #pragma unroll

@@ -356,6 +356,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
   // the centre's column as its owner read it, and each wave's share of the centre's delta
   __shared__ float s_a[TW > 1 ? R * kWave : 1];
   __shared__ float s_da[TW > 1 ? TW : 1][TW > 1 ? R * kWave : 1];
+  __shared__ int s_hands;   // the team waits for its adds before the next token (see below)
   const Shadow shadow = resolve_hot_mode(shadow_arg);
   if (!launch_is_ordered(shadow_arg, shadow)) return;
   const int lane = threadIdx.x & 63;
@@ -432,18 +433,15 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // to the wave of its first position, and occurrence number r of it is worked on in round r
     // (see chain_token_solo).
     int occ = 0, first = lane;
-    bool met = false;   // the word at this lane's position stands in the window (elsewhere)
     {
       unsigned long long m = valid;
       while (m != 0ull) {
         const int l = __builtin_ctzll(m);
         m &= m - 1ull;
-        const int w_l = read_lane(wl, l);
-        if (l < lane && w_l == wl) {
+        if (l < lane && read_lane(wl, l) == wl) {
           if (occ == 0) first = l;
           ++occ;
         }
-        met = met || (l != lane && w_l == wnear_now);
       }
     }
     const bool mine = ok && ((i + first) & (TW - 1)) == wave;
@@ -507,24 +505,20 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // the first columns of this wave are requested before the centre's column is handed round
     unsigned long long mask = __ballot(mine && occ == 0);
     gather(mask);
-    // (worked out here, under the wait for the columns just requested)
-    bool settle = repeats;
-#ifndef W2V_PROBE_NO_HANDOVER
-    if (!settle && unit + 1 < i_end) {
-      const int wn = read_lane(wnear_now, kChainLook + 1);
-      const int nlo = max(nlb, -(i + 1));
-      const int nhi = min(nub, ncols - 2 - i);
-      if (tables.a(wn, d).flags == 0 || nlo < -kChainLook || nhi >= kChainLook - 1) {
-        settle = true;
-      } else {
-        // (most tokens end here: no position that the next window newly reaches holds a word of
-        // this window)
-        const int jn = lane - kChainLook - 1;
-        if (__ballot(met && wl < 0 && jn >= nlo && jn <= nhi && jn != 0) != 0ull)
-          settle = window_hands_over(wl, wnear_now, lane, nlo, nhi, TW);
+    // Whether a column passes to another wave with the next token (window_hands_over): worked
+    // out by one wave that is not the centre's, which would otherwise only wait at the barrier
+    // for the centre's column, from what the token knew when it began, and handed round in LDS.
+    if (wave == ((oa + 1) & (TW - 1))) {
+      bool hands = false;
+      if (!repeats && unit + 1 < i_end) {
+        const int wn = read_lane(wnear_now, kChainLook + 1);
+        const int nlo = max(nlb, -(i + 1));
+        const int nhi = min(nub, ncols - 2 - i);
+        hands = tables.a(wn, d).flags == 0 || nlo < -kChainLook || nhi >= kChainLook - 1 ||
+                window_hands_over(wl, wnear_now, lane, nlo, nhi, TW);
       }
+      if (lane == 0) s_hands = hands ? 1 : 0;
     }
-#endif
     if (wave == oa) {
 #pragma unroll
       for (int r = 0; r < R; ++r) s_a[r * kWave + lane] = a[r];
@@ -555,12 +549,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
     // first position leaves the window), and so may the reader of a word that the next token's
     // window meets again at a new position (window_hands_over), or of any word after a token that
     // is skipped: then this wave's adds have been performed before the team goes on
-#ifdef W2V_PROBE_NO_WAIT
-    if (settle && !repeats) asm volatile("s_nop 0");
-    if (repeats) __builtin_amdgcn_s_waitcnt(0);
-#else
-    if (settle) __builtin_amdgcn_s_waitcnt(0);
-#endif
+    if (repeats || s_hands != 0) __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (wave == oa && tables.written(pa.flags)) {
       zero_col<R>(daa);
