@@ -857,14 +857,14 @@ fold_kernel(float* A, float* B, Shadow shadow, int d) {
 // the n ids of the launch, are left where the update kernels look for "the ids among the 16 most
 // frequent words" and "the most frequent word" (Shadow::hot_seen: four arrays of kHotCountSlots
 // partial counts; the values go to slot 0, the other slots are zeroed); the same for `ids2` (the
-// words read from table A; null: not counted).  The words that are not frequent add about eight
+// words read from table A; null: not counted).  The words that are not frequent add about four
 // ids to every bin (0.4 % of the sample over the kHeavyTop bins, enough to tip a stream that is
 // just below the line): the mean of the other bins is taken off each of the largest.  Two
 // frequent words that share a bin only make the largest bin larger, which errs towards
-// "frequent".  The sample's own noise is 0.13 % of the ids at a share of 6 %.  One workgroup.
+// "frequent".  The sample's own noise is 0.18 % of the ids at a share of 6 %.  One workgroup.
 constexpr int kHeavyThreads = 1024;
 constexpr int kHeavyWaves = kHeavyThreads / kWave;
-constexpr int kHeavySamples = 32768;
+constexpr int kHeavySamples = 16384;
 constexpr int kHeavyPerThread = kHeavySamples / kHeavyThreads;
 constexpr int kHeavyBins = 4096;
 constexpr int kHeavyPerLane = kHeavyBins / kHeavyThreads;   // bins a lane looks after
@@ -939,7 +939,11 @@ count_heavy_kernel(const int* __restrict__ ids, int64_t n, const int* __restrict
           ++binned;
         }
       }
-      if (binned > 0) atomicAdd(&s_binned, binned);
+      // (one LDS atomic per wave, not per thread: a thousand adds to one address take longer than
+      // the histogram)
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) binned += __shfl_xor(binned, m, kWave);
+      if ((tid & 63) == 0 && binned > 0) atomicAdd(&s_binned, binned);
       __syncthreads();
       // every wave picks the largest of its 256 bins, then the first wave the largest of those
       int v[kHeavyPerLane], top[kHeavyTop];
