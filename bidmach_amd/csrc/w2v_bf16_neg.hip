@@ -61,7 +61,6 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
       if (kb + k < nwb) wb[k] = __builtin_amdgcn_readfirstlane(WB[i * nwb + kb + k]);
       if (wb[k] >= 0) {
         load_col16<RP, ALIGNED>(b[k], B + (int64_t)wb[k] * d, lane, d);
-        if (!EVAL && wb[k] < hot.n) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
         if (!EVAL) bscale[k] = scale_of(wb[k], vexp, smode);
       } else {
 #pragma unroll
@@ -69,6 +68,15 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
       }
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) dbb[k][r] = 0.0f;
+    }
+    // (the side columns of the frequent words only now, when every table column has been asked
+    // for: read_side uses what it reads at once, so inside the loop above each frequent column
+    // would be waited for before the next one is requested)
+    if (!EVAL) {
+#pragma unroll
+      for (int k = 0; k < MAXB; ++k) {
+        if (wb[k] >= 0 && wb[k] < hot.n) read_side<RP>(b[k], hot.sb, hot.n, wb[k], lane, d);
+      }
     }
     // the next A column is requested before the current one is written back, so its gather
     // overlaps the exchange; a word that occurs twice among a group's A words is then dotted as
@@ -84,12 +92,23 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
       uint16_t* acol = A + (int64_t)wa * d;
       const bool ahot = !EVAL && wa < hot.n;
       int wanext = -1;
+      // (the next column's side column waits in registers of its own until the column becomes
+      // the current one: added here, it would be waited for before this column's dots; a word
+      // with several side columns keeps the plain way)
+      float anext_side[2 * RP];
+      bool side_pending = false;
       if (j + 1 < nwa) {
         wanext = __builtin_amdgcn_readfirstlane(WA[i * nwa + j + 1]);
         if (wanext >= 0) {
           load_col16<RP, ALIGNED>(anext, A + (int64_t)wanext * d, lane, d);
-          if (!EVAL && wanext < hot.n)
-            read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
+          if (!EVAL && wanext < hot.n) {
+            if (wanext < kTopWords && hot.n >= kTopWords) {
+              read_side<RP>(anext, hot.sa, hot.n, wanext, lane, d);
+            } else {
+              side_col_request<RP>(anext_side, hot.sa + (int64_t)wanext * side_stride(d), lane, d);
+              side_pending = true;
+            }
+          }
         }
       }
       float daa[2 * RP];
@@ -140,6 +159,7 @@ neg_bf16_kernel(int d, int n, int64_t per_wave, int64_t per_wave_ordered, int nw
         wa = wanext;
 #pragma unroll
         for (int r = 0; r < 2 * RP; ++r) a[r] = anext[r];
+        if (side_pending) side_col_add<RP>(a, anext_side);
       }
     }
     if (!EVAL) {

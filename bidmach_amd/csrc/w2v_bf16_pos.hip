@@ -80,11 +80,24 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
     if (j <= hi) load_b(b, wb);
     while (j <= hi) {
       // the next context's column is requested before this one is written back, so its gather
-      // overlaps the exchange -- unless it is the same word again, which has to see this update
+      // overlaps the exchange -- unless it is the same word again, which has to see this update.
+      // (A frequent word's side column waits in registers of its own until the column becomes
+      // the current one: added at once, it would be waited for before this column's dot; a word
+      // with several side columns keeps the plain way.)
       int wbnext = 0;
       const int jnext = next_context(j + 1, wbnext);
       const bool ahead = jnext <= hi && wbnext != wb;
-      if (ahead) load_b(bnext, wbnext);
+      float bnext_side[2 * RP];
+      bool side_pending = false;
+      if (ahead) {
+        if (!EVAL && wbnext < hot.n && !(wbnext < kTopWords && hot.n >= kTopWords)) {
+          load_col16<RP, ALIGNED>(bnext, B + (int64_t)wbnext * d, lane, d);
+          side_col_request<RP>(bnext_side, hot.sb + (int64_t)wbnext * side_stride(d), lane, d);
+          side_pending = true;
+        } else {
+          load_b(bnext, wbnext);
+        }
+      }
       uint16_t* bcol = B + (int64_t)wb * d;
       const bool bhot = !EVAL && wb < hot.n;
       float part = 0.0f;
@@ -111,6 +124,7 @@ pos_bf16_kernel(int d, int n, int64_t per_wave, const int* __restrict__ W,
       if (jnext <= hi && !ahead) load_b(bnext, wbnext);
 #pragma unroll
       for (int r = 0; r < 2 * RP; ++r) b[r] = bnext[r];
+      if (side_pending) side_col_add<RP>(b, bnext_side);
       j = jnext;
       wb = wbnext;
     }
