@@ -27,6 +27,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# w2v_last_launch_form: what the device-side count of a call's word ids decided
+FORM_NAMES = {1: "ordered", 0: "throughput"}
 
 # HBM bytes per launch of the update kernels, measured offline with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE on this same command (summaries under profiles/, named in `source`), scaled by
@@ -237,6 +239,7 @@ class Leg:
                  vexp=0.0, lrate=0.025, mode="train", parts=0, slices=1, head=0):
         from bidmach_amd import corpus
         self.torch, self.name = torch, name
+        self.forms = {}   # which kernels the library took, filled in by run()
         self.cfg = cfg = dict(WORKLOADS[name])
         if tokens > 0:
             cfg["tokens"] = tokens
@@ -288,8 +291,11 @@ class Leg:
         total = self.steps + self.warmup
         return max(self.lrate0 * (1.0 - step / float(max(total, 1))), self.lrate0 * 1e-4)
 
-    def step(self, s, timers=None):
-        from bidmach_amd.cumach import CUMACH, check
+    def step(self, s, timers=None, forms=None):
+        """One pass of both operators over minibatch s.  `forms` (a dict), if given, is told after
+        each of the two calls which kernels the library took for it (w2v_last_launch_form: read
+        back from the device, so it waits for the call)."""
+        from bidmach_amd.cumach import CUMACH, check, load_library
         cfg, A, B, ret, MM = self.cfg, self.A, self.B, self.ret, self.MM
         d, n = cfg["dim"], cfg["tokens"]
         mb, hmb = self.dev_mbs[s % self.ndistinct], self.host_mbs[s % self.ndistinct]
@@ -312,6 +318,8 @@ class Leg:
         if timers:
             timers[0].stop()
             timers[1].start()
+        if forms is not None and not self.evaluating:
+            forms["pos"] = FORM_NAMES.get(load_library().w2v_last_launch_form(), "unknown")
         if self.evaluating:
             check(CUMACH.word2vecEvalNegAsync(d, hmb["G"], cfg["nneg"], cfg["nreuse"], mb["WA"],
                                               mb["WB"], A, B, ret[1:2]), "word2vecEvalNeg")
@@ -329,6 +337,8 @@ class Leg:
                   "word2vecNeg")
         if timers:
             timers[1].stop()
+        if forms is not None and not self.evaluating:
+            forms["neg"] = FORM_NAMES.get(load_library().w2v_last_launch_form(), "unknown")
 
     def finite(self):
         torch = self.torch
@@ -360,6 +370,11 @@ class Leg:
         if self.evaluating:   # reads only: half of the read-and-write model
             pos_b, neg_b = pos_b / 2, neg_b / 2
         assert self.finite(), "tables diverged"
+        # one more, untimed step that asks the library which kernels it takes for this stream
+        self.forms = {}
+        if not self.evaluating:
+            self.step(Wm + K, forms=self.forms)
+            synchronize()
         gbps = lambda b, ms: b / (ms * 1e-3) / 1e9
         return {
             "elapsed": elapsed, "words_per_s": K * cfg["tokens"] / elapsed,
@@ -441,6 +456,8 @@ def brief(leg, r, with_cpu_mbs=0):
            "pos_ms": r["pos_ms"], "neg_ms": r["neg_ms"], "steps": leg.steps,
            "roofline": leg.roofline(r),
            "step_frac_of_hbm_peak": r["step_gbps"] / HBM_PEAK_GBPS}
+    if leg.forms:
+        out["update_kernels_ran"] = dict(leg.forms)
     if with_cpu_mbs:
         out["cpu_baseline"] = leg.cpu(with_cpu_mbs)
         out["cpu_baseline"]["gpu_over_cpu"] = r["words_per_s"] / out["cpu_baseline"]["value"]
@@ -520,6 +537,9 @@ def main():
         "kernels": leg.kernels(r),
         "host_prep_s": leg.prep_s,
     }
+    if leg.forms:
+        # as the library reports it for the step after the timed ones (w2v_last_launch_form)
+        out["config"]["update_kernels_ran"] = dict(leg.forms)
     if not evaluating and not MM and not bf16:
         # which form of the update operators the library took for this stream (its own choice
         # unless --ordered-mode says otherwise): launches full of frequent words run in the
@@ -630,7 +650,8 @@ def extra_legs(torch, lib, args, headline):
         "roofline": leg.roofline(r, m, m["source"]),
         "step_frac_of_hbm_peak": r["step_gbps"] / HBM_PEAK_GBPS,
         "saturated_pair_share": saturated_pair_share(torch, leg.cfg, leg.host_mbs[0], leg.A, leg.B),
-        "ordered_over_throughput_time": headline["ms_per_step"] / r["ms_per_step"]}
+        "ordered_over_throughput_time": headline["ms_per_step"] / r["ms_per_step"],
+        "update_kernels_ran": dict(leg.forms)}
     leg.free()
     lib.w2v_set_ordered_mode(-1)
 

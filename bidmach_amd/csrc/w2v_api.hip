@@ -672,6 +672,26 @@ int w2v_set_ordered_mode(int mode) {
   return 0;
 }
 int w2v_get_ordered_mode(void) { return w2v::get_ordered_mode(); }
+
+int w2v_last_launch_form(void) {
+  const w2v::Shadow* sh = w2v::last_launch_shadow();
+  if (sh == nullptr) return -1;
+  if (sh->ordered == 2) return 1;
+  if (sh->ordered == 0 || sh->hot_total <= 0 || sh->hot_seen == nullptr) return 0;
+  // the counts the kernels of that launch looked at (launch_is_ordered, w2v_device.h)
+  hipStream_t stream = launch_stream(false);
+  int seen[4 * w2v::kHotCountSlots];
+  hipError_t err = hipMemcpyAsync(seen, sh->hot_seen, sizeof(seen), hipMemcpyDeviceToHost, stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  if (err != hipSuccess) return -1;
+  long long sum[4] = {0, 0, 0, 0};
+  for (int t = 0; t < 4; ++t)
+    for (int k = 0; k < w2v::kHotCountSlots; ++k) sum[t] += seen[t * w2v::kHotCountSlots + k];
+  const bool hot_b = w2v::ids_are_hot(sum[0], sum[1], sh->hot_total);
+  const bool hot_a =
+      sh->hot_total_a > 0 ? w2v::ids_are_hot(sum[2], sum[3], sh->hot_total_a) : hot_b;
+  return (hot_a || hot_b) ? 1 : 0;
+}
 int w2v_set_ordered_workers(int pos_workers, int neg_workers) {
   if (pos_workers < 0 || neg_workers < 0) return (int)hipErrorInvalidValue;
   w2v::set_ordered_workers(pos_workers, neg_workers);

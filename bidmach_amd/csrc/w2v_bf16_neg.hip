@@ -228,6 +228,7 @@ hipError_t launch(hipStream_t stream, int d, int n, int nwa, int nwb, const int*
       // kernel whatever the launch holds, on the ordered form's number of workers
       if (!neg_rows_bf16_available(d, nwa)) return hipErrorInvalidValue;
       shadow.ordered = 2;
+      note_last_launch(shadow);
     }
     rows = shadow.ordered != 0 && neg_rows_bf16_available(d, nwa);
     if (shadow.ordered != 0 && !rows) {

@@ -303,7 +303,7 @@ __device__ __forceinline__ long long sum_hot_counts(const int* part) {
 // `zero` of them of the most frequent one, are full of frequent words: the 16 most frequent are a
 // sixteenth of all, or the most frequent alone is a 48th (its atomics retire one after the other,
 // and at 5 ids per group a 48th of them already lasts about half as long as the whole pass).
-__device__ __forceinline__ bool ids_are_hot(long long low, long long zero, long long total) {
+__host__ __device__ __forceinline__ bool ids_are_hot(long long low, long long zero, long long total) {
   return low * kHotShareDen >= total || zero * kHotZeroShareDen >= total;
 }
 

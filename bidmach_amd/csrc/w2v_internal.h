@@ -57,6 +57,11 @@ size_t occurs_bytes();
 hipError_t prepare_hot_mode(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
                             int64_t n2, const float* A, const float* B, int d, int64_t nwg,
                             int waves_per_wg, Shadow* shadow);
+// What prepare_hot_mode left for the calling thread's most recent update launch (the counters it
+// points to are the launch's own until the thread's next update launch): for w2v_last_launch_form.
+// Null before the thread's first update launch.
+const Shadow* last_launch_shadow();
+void note_last_launch(const Shadow& shadow);
 // The same for a sliced model, whose shadowed columns are the first columns of part 0.
 hipError_t prepare_hot_mode_sliced(hipStream_t stream, const int* ids, int64_t n, const int* ids2,
                                    int64_t n2, const SliceMap& m, int d, int64_t nwg,

@@ -1127,6 +1127,15 @@ int get_hot_update_mode() { return g_hot_update_mode.load(); }
 // invisible to each other anyway; with the Zipf share of the top word that is several hundred
 // invisible updates of that word per 2048 waves.  Below that size the exact mode is used.
 constexpr int64_t kCombineMinWaves = 2048;
+
+static thread_local Shadow t_last_launch{};
+static thread_local bool t_last_launch_set = false;
+const Shadow* last_launch_shadow() { return t_last_launch_set ? &t_last_launch : nullptr; }
+void note_last_launch(const Shadow& shadow) {
+  t_last_launch = shadow;
+  t_last_launch_set = true;
+}
+
 template <class Tables>
 static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64_t n,
                                        const int* ids2, int64_t n2, const Tables& tables,
@@ -1146,7 +1155,10 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   shadow->grid_c = g_ordered_copies.load();
   shadow->grid_r = g_ordered_twins.load();
   if (shadow->combine != kHotCombining) shadow->pub_a = shadow->pub_b = nullptr;
-  if (n <= 0 || (forced && shadow->pub_a == nullptr)) return hipSuccess;
+  if (n <= 0 || (forced && shadow->pub_a == nullptr)) {
+    note_last_launch(*shadow);
+    return hipSuccess;
+  }
   // Shadow copies pay only if the launch really holds hot words: count them first (the kernels
   // read the count from memory, the host does not wait for it).  The same pass notes which hot
   // ids occur at all, for the read copies.
@@ -1161,6 +1173,7 @@ static hipError_t prepare_hot_mode_for(hipStream_t stream, const int* ids, int64
   if (shadow->pub_a != nullptr)
     hipLaunchKernelGGL(publish_kernel, dim3(kHotWords, 2), dim3(kBlock), 0, stream, A, B, *shadow,
                        d);
+  note_last_launch(*shadow);
   return hipGetLastError();
 }
 

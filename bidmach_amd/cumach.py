@@ -75,6 +75,7 @@ SYMBOLS = {
     "w2v_get_max_workgroups": (_I, []),
     "w2v_set_ordered_mode": (_I, [_I]),
     "w2v_get_ordered_mode": (_I, []),
+    "w2v_last_launch_form": (_I, []),
     "w2v_set_ordered_workers": (_I, [_I, _I]),
     "w2v_set_ordered_copies": (_I, [_I, _I]),
     "w2v_set_hot_update_mode": (_I, [_I]),

@@ -233,6 +233,12 @@ int w2v_get_max_workgroups(void);
  *   0  never;  1  always. */
 int w2v_set_ordered_mode(int mode);
 int w2v_get_ordered_mode(void);
+/* Which form the calling thread's most recent update call (any of the operators above) took: 1
+ * the ordered form, 0 the throughput kernels, -1 if the thread has made no update call yet (or
+ * the counts could not be read).  Waits for the thread's launch stream and reads back the counts
+ * that the kernels of that launch looked at; for logs and benchmarks, not for a training loop.
+ * No counterpart in the reference. */
+int w2v_last_launch_form(void);
 /* Number of wavefronts (workers) the ordered form of word2vecPos and of word2vecNeg / NegFilt
  * spreads a launch over; 0 = the library's own numbers (the default).  Fewer workers follow the
  * sequential order more closely and take longer; w2v_set_max_workgroups bounds them as well. */

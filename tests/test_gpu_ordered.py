@@ -359,3 +359,41 @@ def test_one_worker_reproduces_the_sequential_sliced_passes(gpu, oracle, islice,
     assert err <= 2e-5, err
     _, loose = run(0)
     assert max(np.abs(g - h).max() for g, h in zip(loose, host)) > 50 * err + 1e-3
+
+
+def test_last_launch_form_reports_what_the_device_decided(gpu, oracle):
+    """w2v_last_launch_form reads back the counts that the kernels of the thread's last update
+    call looked at: a launch over a handful of words took the ordered form, a launch of distinct
+    words the throughput kernels, and forcing either way is reported as forced."""
+    torch, CUMACH = gpu
+    from bidmach_amd.cumach import load_library
+    lib = load_library()
+    rng = np.random.default_rng(5)
+    d, skip, n = 64, 3, 4000
+    LB, UB = corpus.window_bounds(n, skip, rng)
+    A = (rng.standard_normal((n + 16, d)) * 0.1).astype(np.float32)
+    B = (rng.standard_normal((n + 16, d)) * 0.1).astype(np.float32)
+    few = rng.integers(0, 6, n).astype(np.int32)
+    distinct = (16 + rng.permutation(n)).astype(np.int32)
+    parity.gpu_pos(gpu, d, skip, few, LB, UB, A, B, 0.01, 0.0)
+    assert lib.w2v_last_launch_form() == 1
+    parity.gpu_pos(gpu, d, skip, distinct, LB, UB, A, B, 0.01, 0.0)
+    assert lib.w2v_last_launch_form() == 0
+    G = n // 5
+    parity.gpu_neg(gpu, d, G, 5, 5, few[:5 * G], distinct[:5 * G], A, B, 0.01, 0.0)
+    assert lib.w2v_last_launch_form() == 1          # the A words are the frequent ones here
+    parity.gpu_neg(gpu, d, G, 5, 5, distinct[:5 * G], distinct[::-1][:5 * G].copy(), A, B, 0.01, 0.0)
+    assert lib.w2v_last_launch_form() == 0
+    lib.w2v_set_ordered_mode(1)
+    try:
+        parity.gpu_pos(gpu, d, skip, distinct, LB, UB, A, B, 0.01, 0.0)
+        assert lib.w2v_last_launch_form() == 1
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+    lib.w2v_set_ordered_mode(0)
+    try:
+        parity.gpu_pos(gpu, d, skip, few, LB, UB, A, B, 0.01, 0.0)
+        assert lib.w2v_last_launch_form() == 0
+    finally:
+        lib.w2v_set_ordered_mode(-1)
+
