@@ -98,7 +98,7 @@ neg_rows_kernel(int d, int ngroups, int idlimit, int nwa, int nwb, int64_t per_c
           pre = (lane == j) ? s : pre;
         }
       }
-      const float gl = -lrate * sat_sigmoid(pre);
+      const float gl = -lrate * sat_sigmoid_fast(pre);
       const float bs = read_lane(sbl, k);
       float dbb[R];
       zero_col<R>(dbb);

@@ -320,7 +320,7 @@ __device__ __forceinline__ void chain_token_solo(int i, int wi, int jlo, int jhi
             pre = (lane == c) ? s : pre;
           }
         }
-        const float gl = lrate * (1.0f - sat_sigmoid(pre));
+        const float gl = lrate * (1.0f - sat_sigmoid_fast(pre));
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
           if (c < n) {
@@ -485,7 +485,7 @@ pos_chain_kernel(int d, int ncols, int64_t per_chain, const int* __restrict__ W,
           pre = (lane == c) ? s : pre;
         }
       }
-      const float gl = lrate * (1.0f - sat_sigmoid(pre));
+      const float gl = lrate * (1.0f - sat_sigmoid_fast(pre));
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         if (c < n) {
